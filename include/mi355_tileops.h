@@ -1,0 +1,129 @@
+/*
+ * mi355_tileops.h -- C ABI of the MI355X (gfx950) paged GQA decode library.
+ *
+ * Plain pointers and sizes only; every entry point enqueues work on the given HIP stream and returns.
+ * No entry point synchronises the device, reads device memory on the host, or allocates device memory:
+ * the caller owns inputs, output and workspace.  All functions return 0 on success or a negative
+ * MI355_E* code; mi355_last_error() then gives a thread-local message.  Nothing throws or aborts.
+ *
+ * The reference (tile-ai/TileOPs) has no native ABI: its kernels are TileLang programs JIT-compiled to
+ * CUDA and reached through torch custom ops.  Each declaration below cites the reference interface whose
+ * job it takes over.
+ */
+#ifndef MI355_TILEOPS_H
+#define MI355_TILEOPS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_ABI_VERSION 1
+
+/* element types */
+#define MI355_DT_BF16 0
+#define MI355_DT_FP16 1
+#define MI355_DT_FP8_E4M3FN 2 /* OCP e4m3fn (gfx950 native); KV cache only */
+
+/* kernel selection for mi355_gqa_paged_decode(): which implementation serves the call */
+#define MI355_KERNEL_AUTO 0    /* MFMA kernel when the shape qualifies, else the generic one */
+#define MI355_KERNEL_GENERIC 1 /* VALU kernel: any head_dim in {64,128,256}, any page size, any group */
+#define MI355_KERNEL_MFMA 2    /* MFMA kernel; MI355_EUNSUPPORTED if the shape does not qualify */
+
+/* error codes */
+#define MI355_OK 0
+#define MI355_EINVAL (-1)       /* an argument violates the contract (message names it) */
+#define MI355_EUNSUPPORTED (-2) /* legal call, but no kernel in this library serves it */
+#define MI355_EWORKSPACE (-3)   /* workspace pointer missing or too small */
+#define MI355_ELAUNCH (-4)      /* HIP reported an error at launch */
+#define MI355_EDEVICE (-5)      /* current device is not gfx950 */
+
+/* Version of this ABI (MI355_ABI_VERSION of the library that was loaded). */
+int mi355_abi_version(void);
+
+/* Message for the last error on the calling thread ("" if none). The pointer stays valid until the
+ * next failing call on the same thread. */
+const char* mi355_last_error(void);
+
+/*
+ * Workspace requirement and split plan for one decode call of the given shape.
+ *
+ * Replaces the host prologue of GQADecodePagedKernel.forward
+ * (src/tileops/kernels/attention/gqa_decode_paged.py:683-721), which reads max(real_seqlen_kv) back to
+ * the host, builds split_length with torch ops and allocates glse / Output_partial per call.  Here the
+ * plan depends only on shapes, so nothing is read back; the per-sequence split bounds are derived from
+ * real_seqlen_kv inside the kernels.
+ *
+ *   max_blocks_per_seq : width of block_table actually usable (>= ceil(max context / page_size))
+ *   num_split_in       : 0 = choose; > 0 = upper bound on KV splits per sequence (generic kernel) /
+ *                        ignored by the MFMA kernel, which partitions the KV tile stream evenly over
+ *                        all compute units instead
+ *   kernel             : MI355_KERNEL_*
+ * Outputs: *workspace_bytes (may be 0), *num_split_out (splits per sequence the generic kernel will
+ * use at most; number of stream partitions for the MFMA kernel), *kernel_out (the kernel AUTO resolved to).
+ */
+int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                                     int64_t max_blocks_per_seq, int q_dtype, int kv_dtype, int num_split_in,
+                                     int kernel, size_t* workspace_bytes, int* num_split_out, int* kernel_out);
+
+/*
+ * Paged GQA decode attention, one call = one forward of
+ * GroupedQueryAttentionDecodePagedWithKVCacheFwdOp
+ * (src/tileops/ops/attention/gqa.py:1443-1454 -> GQADecodePagedKernel.forward,
+ *  src/tileops/kernels/attention/gqa_decode_paged.py:669-746; custom-op argument lists :401-421, :451-475),
+ * i.e. the reference's no-split kernel (:75-168), split kernel (:209-342) and combine (:344-374).
+ *
+ *   q            [batch, q_len, heads, dim]  q_dtype (bf16|fp16), contiguous.  q_len == 1 is the reference op.
+ *   k, v         [n_phys_tokens, heads_kv, dim]  kv_dtype, contiguous: the physical page pool,
+ *                page p = tokens [p*page_size, (p+1)*page_size)
+ *   k_scale,
+ *   v_scale      [n_phys_tokens, heads_kv] fp32 per-token-per-head dequant scales (x = fp8 * scale);
+ *                required iff kv_dtype == MI355_DT_FP8_E4M3FN, else NULL
+ *                (format of src/tileops/kernels/fp8_quant.py:44-60; dequant as kernels/attention/gqa_fwd.py:1063-1065)
+ *   seqlens      [batch] int32: tokens of context per sequence, INCLUDING the q_len new tokens
+ *   block_table  [batch, >= ceil(seqlens[b]/page_size)] int32 physical page ids, row stride bt_row_stride (elements)
+ *   out          [batch, q_len, heads, dim] q_dtype
+ *   workspace    >= the size mi355_gqa_paged_decode_workspace() reports for the same arguments, 256-byte aligned
+ *   sm_scale     softmax scale applied to q.k  (the op passes dim**-0.5 unless overridden, gqa.py:81-82)
+ *   softcap      0 = off, else scores := softcap * tanh(scores / softcap)  (online_softmax.py:153-173)
+ *   causal       with q_len > 1: query i sees key j iff j <= i + (seqlens[b] - q_len)  (gqa.py:558-562)
+ *   num_split    as num_split_in above;  kernel as above
+ *
+ * Sequences with seqlens[b] == 0 produce zeros.  Tokens not addressed by (block_table, seqlens) are never read.
+ */
+int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const float* k_scale,
+                           const float* v_scale, const int32_t* seqlens, const int32_t* block_table,
+                           int64_t bt_row_stride, void* out, void* workspace, size_t workspace_bytes, int batch,
+                           int q_len, int heads, int heads_kv, int dim, int page_size, int64_t n_phys_tokens,
+                           int q_dtype, int kv_dtype, float sm_scale, float softcap, int causal, int num_split,
+                           int kernel, void* hip_stream);
+
+/*
+ * Index-probe: materialise the logical KV rows a decode call would read, with the same device page
+ * arithmetic the attention kernels use.  dense_out [batch, max_len, heads_kv * dim] elem_bytes-wide
+ * elements; rows t >= seqlens[b] are left untouched.  Lets a test compare the gather bit-for-bit with
+ * k.view(P, page, H_kv, D)[block_table[b, :n]] -- the page reassembly of the reference's ref_program
+ * (tests/ops/attention/test_gqa_decode_paged.py:46-59).
+ */
+int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
+                       void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size,
+                       int64_t n_phys_tokens, void* hip_stream);
+
+/*
+ * Append one new token per sequence to a paged FP8 cache: per-(token, kv-head) absmax/448 scale,
+ * clamp(x/scale, +-448) -> e4m3fn (round-to-nearest-even), written at logical position seqlens[b]-1.
+ * Takes over the per-token quantizer FP8QuantKernel (src/tileops/kernels/fp8_quant.py:14-64) fused with
+ * the page append of the paged prefill kernel (src/tileops/kernels/attention/gqa_fwd.py:1124-1168).
+ *   x_new [batch, heads_kv, dim] x_dtype (bf16|fp16); cache [n_phys_tokens, heads_kv, dim] fp8;
+ *   scale [n_phys_tokens, heads_kv] fp32.
+ */
+int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int32_t* seqlens,
+                        const int32_t* block_table, int64_t bt_row_stride, int batch, int heads_kv, int dim,
+                        int page_size, int64_t n_phys_tokens, int x_dtype, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_TILEOPS_H */

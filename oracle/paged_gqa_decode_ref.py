@@ -1,0 +1,244 @@
+"""TEST INFRASTRUCTURE ONLY -- CPU restatement of the reference's paged GQA decode semantics.
+
+Nothing under ``tileops_amd/`` may import this module.  Only ``tests/``, ``__graft_entry__.smoke()`` and
+``bench.py``'s ``cpu_baseline`` leg use it, and only as the checker.
+
+Every function cites the reference file:line it follows (paths relative to the reference checkout).
+
+Parity status of each function (how it is pinned, without importing the reference):
+
+* ``gather_pages``              pure indexing; pinned bit-exact against ``k.view(P, page, H_kv, D)[table]``
+                                and by a per-token loop restating ``_physical_pos``.
+* ``ref_paged_gqa_decode``      pinned against ``torch.nn.functional.scaled_dot_product_attention`` (a library
+                                routine, the reference benchmark's own baseline), a float64 NumPy brute force,
+                                and closed forms (q=0 -> mean of V, len=1 -> V row, dominant key, softcap->inf).
+* ``ref_gqa_decode_contiguous`` pinned against SDPA and the paged oracle with an identity table.
+* ``quantize_kv_per_token``     pinned against the C codec in ``oracle/fp8_e4m3fn.c`` and torch's fp8 cast.
+* causal chunk mask             pinned by "query i of a chunk == single-token decode at length len-S_q+i+1".
+
+The exact floating-point bits of the reference's TileLang-generated CUDA kernels are not reproducible here
+(TileLang is absent); the reference itself defines correctness against this torch program within tolerance.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import numpy as np
+import torch
+
+FP8_MAX = 448.0
+
+
+def physical_pos(block_table: torch.Tensor, batch_idx: int, logical_pos: int, page_size: int) -> int:
+    """Logical token -> physical token.  tests/ops/attention/test_gqa_prefill_paged.py:25-31."""
+    page = int(block_table[batch_idx, logical_pos // page_size])
+    return page * page_size + logical_pos % page_size
+
+
+def gather_pages(
+    cache: torch.Tensor, block_table_row: torch.Tensor, length: int, page_size: int
+) -> torch.Tensor:
+    """Reassemble one sequence's logical ``[length, ...]`` rows from the physical pool ``[N_kv, ...]``.
+
+    tests/ops/attention/test_gqa_decode_paged.py:46-59 (page-by-page copy, then truncate to the real
+    length).  Pure indexing: the result is bit-identical to the pool rows it names.
+    """
+    if length == 0:
+        return cache[:0]
+    n_pages = math.ceil(length / page_size)
+    pages = block_table_row[:n_pages].to(torch.long)
+    idx = (pages[:, None] * page_size + torch.arange(page_size)[None, :]).reshape(-1)[:length]
+    return cache.index_select(0, idx)
+
+
+def _scores_to_probs(scores: torch.Tensor, softcap: float) -> torch.Tensor:
+    if softcap > 0:
+        # tests/ops/attention/test_gqa_decode_paged.py:66-67 ; online_softmax.py:162-171
+        scores = softcap * torch.tanh(scores / softcap)
+    return scores
+
+
+def ref_paged_gqa_decode(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    real_seqlen_kv: torch.Tensor,
+    block_table: torch.Tensor,
+    *,
+    page_size: int,
+    sm_scale: Optional[float] = None,
+    softcap: float = 0.0,
+    k_scale: Optional[torch.Tensor] = None,
+    v_scale: Optional[torch.Tensor] = None,
+    is_causal: bool = True,
+    out_dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """fp32 attention over gathered (and dequantized) pages, cast to ``q.dtype``.
+
+    ``q`` is ``[B, H, D]`` (one query token; tests/ops/attention/test_gqa_decode_paged.py:30-72) or
+    ``[B, S_q, H, D]`` (a chunk of S_q new tokens whose K/V are already in the cache; the mask is
+    bottom-right aligned -- key j visible to query i iff ``j <= i + (len - S_q)`` --
+    tests/ops/attention/test_gqa_prefill_paged.py:110-115, src/tileops/ops/attention/gqa.py:558-562).
+    ``k, v`` are the physical pools ``[N_kv, H_kv, D]`` in fp16/bf16/fp32 or float8_e4m3fn; with fp8 the
+    per-token-per-head fp32 ``k_scale, v_scale [N_kv, H_kv]`` dequantize as ``fp8.float() * scale``
+    (tests/ops/attention/test_gqa_fp8.py:216-219).
+
+    Uses a grouped einsum instead of the reference's ``repeat_interleave`` head expansion: same numbers,
+    no ``group``-fold copy of K/V.
+    """
+    multi = q.dim() == 4
+    q4 = q if multi else q.unsqueeze(1)
+    B, S_q, H, D = q4.shape
+    H_kv = k.shape[1]
+    G = H // H_kv
+    scale = D ** -0.5 if sm_scale is None else sm_scale
+    out = torch.empty(B, S_q, H, D, dtype=torch.float32)
+    for b in range(B):
+        n = int(real_seqlen_kv[b])
+        if n == 0:
+            out[b] = 0.0  # softmax over nothing: nan_to_num convention, test_gqa_prefill_paged.py:115
+            continue
+        k_b = gather_pages(k, block_table[b], n, page_size).float()
+        v_b = gather_pages(v, block_table[b], n, page_size).float()
+        if k_scale is not None:
+            k_b = k_b * gather_pages(k_scale, block_table[b], n, page_size).float()[..., None]
+        if v_scale is not None:
+            v_b = v_b * gather_pages(v_scale, block_table[b], n, page_size).float()[..., None]
+        qg = q4[b].float().reshape(S_q, H_kv, G, D)
+        scores = torch.einsum("sjgd,njd->jgsn", qg, k_b) * scale  # [H_kv, G, S_q, n]
+        scores = _scores_to_probs(scores, softcap)
+        if multi and is_causal and S_q > 1:
+            q_pos = torch.arange(S_q)[:, None] + (n - S_q)
+            kv_pos = torch.arange(n)[None, :]
+            scores = scores.masked_fill(~(kv_pos <= q_pos), float("-inf"))
+        probs = torch.softmax(scores, dim=-1).nan_to_num()
+        o = torch.einsum("jgsn,njd->sjgd", probs, v_b)
+        out[b] = o.reshape(S_q, H, D)
+    out = out.to(out_dtype or q.dtype)
+    return out if multi else out.squeeze(1)
+
+
+def ref_gqa_decode_contiguous(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    sm_scale: Optional[float] = None,
+    softcap: float = 0.0,
+) -> torch.Tensor:
+    """Contiguous-cache GQA decode: ``q [B,H,D]``, ``k,v [B,S,H_kv,D]``.  workloads/attention/gqa.py:165-175."""
+    B, H, D = q.shape
+    H_kv = k.shape[2]
+    G = H // H_kv
+    scale = D ** -0.5 if sm_scale is None else sm_scale
+    qg = q.float().reshape(B, H_kv, G, D)
+    scores = torch.einsum("bjgd,bnjd->bjgn", qg, k.float()) * scale
+    scores = _scores_to_probs(scores, softcap)
+    probs = torch.softmax(scores, dim=-1)
+    o = torch.einsum("bjgn,bnjd->bjgd", probs, v.float())
+    return o.reshape(B, H, D).to(q.dtype).contiguous()
+
+
+def brute_force_f64(
+    q: np.ndarray,
+    k: np.ndarray,
+    v: np.ndarray,
+    lens: np.ndarray,
+    table: np.ndarray,
+    page_size: int,
+    sm_scale: float,
+    softcap: float = 0.0,
+    causal: bool = True,
+) -> np.ndarray:
+    """Token-by-token float64 evaluation (tiny shapes only).  Same semantics as ``ref_paged_gqa_decode``
+    written with scalar page arithmetic so an indexing slip in either shows up as a mismatch."""
+    multi = q.ndim == 4
+    q4 = q if multi else q[:, None]
+    B, S_q, H, D = q4.shape
+    H_kv = k.shape[1]
+    G = H // H_kv
+    out = np.zeros((B, S_q, H, D), dtype=np.float64)
+    for b in range(B):
+        n = int(lens[b])
+        for s in range(S_q):
+            limit = n - S_q + s + 1 if (multi and causal) else n
+            for h in range(H):
+                j = h // G
+                sc = np.empty(max(limit, 0), dtype=np.float64)
+                rows = np.empty((max(limit, 0), D), dtype=np.float64)
+                for t in range(limit):
+                    phys = int(table[b, t // page_size]) * page_size + t % page_size
+                    x = float(np.dot(q4[b, s, h].astype(np.float64), k[phys, j].astype(np.float64))) * sm_scale
+                    if softcap > 0:
+                        x = softcap * math.tanh(x / softcap)
+                    sc[t] = x
+                    rows[t] = v[phys, j]
+                if limit <= 0:
+                    continue
+                p = np.exp(sc - sc.max())
+                p /= p.sum()
+                out[b, s, h] = p @ rows
+    return out if multi else out[:, 0]
+
+
+def quantize_kv_per_token(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-(token, kv-head) FP8-E4M3FN quantizer: ``x [N, H_kv, D]`` -> ``(q8 [N,H_kv,D] fp8, scale [N,H_kv] f32)``.
+
+    workloads/fp8_quant.py:27-33: ``amax = |x|.amax(-1).clamp(min=1e-4)``; ``scale = amax / 448``;
+    ``q = clamp(x / scale, -448, 448).to(float8_e4m3fn)``.  The clamp matters: torch's cast does not
+    saturate (values rounding above 448 become NaN).
+    """
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1, keepdim=True).clamp(min=1e-4)
+    scale = amax / FP8_MAX
+    q8 = torch.clamp(xf / scale, min=-FP8_MAX, max=FP8_MAX).to(torch.float8_e4m3fn)
+    return q8, scale.squeeze(-1).contiguous()
+
+
+def dequantize_kv(q8: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """``fp8.float() * scale``.  tests/ops/attention/test_gqa_fp8.py:216-219."""
+    return q8.float() * scale.float()[..., None]
+
+
+# --- split-KV bookkeeping restated from the reference (known-answer material for the host-side tests) ----
+
+
+def reference_block_ns(page_size: int) -> tuple[int, ...]:
+    """Tile heights the reference's generic paged kernel accepts.
+    src/tileops/kernels/attention/gqa_decode_paged.py:21-33."""
+    if page_size <= 0:
+        raise ValueError("page_size must be positive")
+    ns = tuple(n for n in (128, 64) if n <= page_size and page_size % n == 0)
+    if ns:
+        return ns
+    if page_size < 64:
+        return (page_size,)
+    raise ValueError(f"page_size={page_size} matches no supported block_N")
+
+
+def combine_partials(partial_o: torch.Tensor, lse2: torch.Tensor) -> torch.Tensor:
+    """Merge normalised per-split outputs with their log2-domain LSE.
+
+    src/tileops/kernels/attention/gqa_decode_paged.py:344-374:
+    ``lse = log2 sum_s 2^(lse_s - max) + max`` ; ``O = sum_s 2^(lse_s - lse) * O_s``.
+    ``partial_o [..., S, D]``, ``lse2 [..., S]`` (``-inf`` marks an empty split).
+    """
+    m = lse2.max(dim=-1, keepdim=True).values
+    m = torch.where(torch.isfinite(m), m, torch.zeros_like(m))
+    w = torch.exp2(lse2 - m)
+    lse = torch.log2(w.sum(dim=-1, keepdim=True)) + m
+    wn = torch.exp2(lse2 - lse).nan_to_num()
+    return (partial_o * wn[..., None]).sum(dim=-2)
+
+
+def reference_roofline(
+    batch: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int, page_size: int, elem_bytes: int
+) -> tuple[int, int]:
+    """(flops, bytes) exactly as src/tileops/perf/formulas.py:690-711 (S = pool size, K/V counted once)."""
+    flops = 4 * batch * heads * seqlen_kv * dim
+    q_elems = batch * heads * dim
+    kv_elems = seqlen_kv * heads_kv * dim
+    meta = batch * 4 + batch * max(1, (seqlen_kv + page_size - 1) // page_size) * 4
+    return int(flops), int((q_elems + 2 * kv_elems + q_elems) * elem_bytes + meta)

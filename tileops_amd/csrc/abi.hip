@@ -1,0 +1,231 @@
+// extern "C" entry points of libmi355_tileops: argument validation, kernel choice, launch.
+// Never throws, never aborts, never synchronises, never allocates device memory.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.h"
+
+using namespace mi355;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool is_q_dtype(int d) { return d == MI355_DT_BF16 || d == MI355_DT_FP16; }
+bool is_kv_dtype(int d) { return d == MI355_DT_BF16 || d == MI355_DT_FP16 || d == MI355_DT_FP8_E4M3FN; }
+
+// Shape-only checks shared by the workspace query and the launch.
+int check_shape(int batch, int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype) {
+  if (batch < 0) return fail(MI355_EINVAL, "batch must be non-negative, got %d", batch);
+  if (q_len <= 0) return fail(MI355_EINVAL, "q_len must be positive, got %d", q_len);
+  if (heads <= 0) return fail(MI355_EINVAL, "heads must be positive, got %d", heads);
+  if (heads_kv <= 0) return fail(MI355_EINVAL, "heads_kv must be positive, got %d", heads_kv);
+  if (heads % heads_kv != 0) return fail(MI355_EINVAL, "heads must be divisible by heads_kv (%d %% %d)", heads, heads_kv);
+  if (dim <= 0) return fail(MI355_EINVAL, "dim must be positive, got %d", dim);
+  if (page_size <= 0) return fail(MI355_EINVAL, "page_size must be positive, got %d", page_size);
+  if (!is_q_dtype(q_dtype)) return fail(MI355_EINVAL, "q_dtype must be bf16 or fp16, got code %d", q_dtype);
+  if (!is_kv_dtype(kv_dtype)) return fail(MI355_EINVAL, "kv_dtype must be bf16, fp16 or fp8_e4m3fn, got code %d", kv_dtype);
+  if (kv_dtype != MI355_DT_FP8_E4M3FN && kv_dtype != q_dtype)
+    return fail(MI355_EINVAL, "a 16-bit kv_dtype must equal q_dtype (q code %d, kv code %d)", q_dtype, kv_dtype);
+  if (dim != 64 && dim != 128 && dim != 256)
+    return fail(MI355_EUNSUPPORTED, "head dim %d is not served (64, 128 or 256)", dim);
+  if (batch > 65535) return fail(MI355_EUNSUPPORTED, "batch %d exceeds 65535", batch);
+  return MI355_OK;
+}
+
+struct Plan {
+  int kernel;        // MI355_KERNEL_GENERIC or MI355_KERNEL_MFMA
+  int max_splits;    // generic
+  int split_tokens;  // generic
+  int n_parts;       // mfma
+  size_t part_o_bytes, part_lse_bytes;
+};
+
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_size, int64_t max_blocks_per_seq, int q_dtype,
+              int kv_dtype, float softcap, int num_split_in, int kernel, Plan* plan) {
+  if (max_blocks_per_seq < 0) return fail(MI355_EINVAL, "max_blocks_per_seq must be non-negative");
+  if (num_split_in < 0) return fail(MI355_EINVAL, "num_split must be non-negative, got %d", num_split_in);
+  const int rows = q_len * (heads / heads_kv);
+  bool mfma_ok = mfma_supported(q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype, softcap);
+  if (kernel == MI355_KERNEL_MFMA && !mfma_ok)
+    return fail(MI355_EUNSUPPORTED, "the MFMA kernel does not serve this shape (dim %d, page_size %d, rows %d, dtypes %d/%d)",
+                dim, page_size, rows, q_dtype, kv_dtype);
+  if (kernel != MI355_KERNEL_AUTO && kernel != MI355_KERNEL_GENERIC && kernel != MI355_KERNEL_MFMA)
+    return fail(MI355_EINVAL, "unknown kernel selector %d", kernel);
+  plan->kernel = (kernel == MI355_KERNEL_GENERIC || !mfma_ok) ? MI355_KERNEL_GENERIC : MI355_KERNEL_MFMA;
+  if (plan->kernel == MI355_KERNEL_GENERIC) {
+    // Fixed-length splits of ~512 tokens, at most 64 per sequence, bounded by what the table can address.
+    plan->split_tokens = 512;
+    int64_t max_ctx = max_blocks_per_seq * (int64_t)page_size;
+    int64_t cap = (max_ctx + plan->split_tokens - 1) / plan->split_tokens;
+    if (cap < 1) cap = 1;
+    int ms = num_split_in > 0 ? num_split_in : 64;
+    if (ms > 1024) ms = 1024;
+    if (ms > cap) ms = (int)cap;
+    plan->max_splits = ms;
+    plan->n_parts = 0;
+    size_t slots = (size_t)batch * ms;
+    plan->part_o_bytes = ms > 1 ? align256(slots * heads_kv * rows * dim * sizeof(float)) : 0;
+    plan->part_lse_bytes = ms > 1 ? align256(slots * heads_kv * rows * sizeof(float)) : 0;
+  } else {
+    plan->max_splits = 0;
+    plan->split_tokens = 0;
+    plan->n_parts = mfma_num_parts(heads_kv, rows, kv_dtype);
+    size_t total = mfma_workspace_bytes(plan->n_parts, heads_kv, rows, dim);
+    plan->part_o_bytes = total;  // the MFMA launcher lays out its own workspace
+    plan->part_lse_bytes = 0;
+  }
+  return MI355_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_abi_version(void) { return MI355_ABI_VERSION; }
+
+const char* mi355_last_error(void) { return g_err; }
+
+int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                                     int64_t max_blocks_per_seq, int q_dtype, int kv_dtype, int num_split_in, int kernel,
+                                     size_t* workspace_bytes, int* num_split_out, int* kernel_out) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
+  if (rc) return rc;
+  Plan plan;
+  // softcap does not change the plan; the MFMA kernel serves both settings
+  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in, kernel,
+                 &plan);
+  if (rc) return rc;
+  if (workspace_bytes) *workspace_bytes = plan.part_o_bytes + plan.part_lse_bytes;
+  if (num_split_out) *num_split_out = plan.kernel == MI355_KERNEL_GENERIC ? plan.max_splits : plan.n_parts;
+  if (kernel_out) *kernel_out = plan.kernel;
+  return MI355_OK;
+}
+
+int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                           const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out, void* workspace,
+                           size_t workspace_bytes, int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                           int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale, float softcap, int causal,
+                           int num_split, int kernel, void* hip_stream) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
+  if (rc) return rc;
+  if (batch == 0) return MI355_OK;
+  if (!q || !k || !v || !seqlens || !block_table || !out)
+    return fail(MI355_EINVAL, "q, k, v, seqlens, block_table and out must be non-null");
+  const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
+  if (fp8 && (!k_scale || !v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale are required with an fp8 KV cache");
+  if (!fp8 && (k_scale || v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale must be null unless kv_dtype is fp8_e4m3fn");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens,
+                page_size);
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (!(softcap >= 0.f)) return fail(MI355_EINVAL, "softcap must be non-negative");
+  if (!(sm_scale == sm_scale)) return fail(MI355_EINVAL, "sm_scale is NaN");
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
+    return fail(MI355_EINVAL, "q, k, v and out must be 16-byte aligned");
+  Plan plan;
+  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan);
+  if (rc) return rc;
+  const size_t need = plan.part_o_bytes + plan.part_lse_bytes;
+  if (need > 0) {
+    if (!workspace) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got null", need);
+    if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
+  }
+
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.seqlens = seqlens;
+  p.block_table = block_table;
+  p.bt_row_stride = bt_row_stride;
+  p.out = out;
+  p.part_o = (float*)workspace;
+  p.part_lse = (float*)((char*)workspace + plan.part_o_bytes);
+  p.batch = batch;
+  p.q_len = q_len;
+  p.heads = heads;
+  p.heads_kv = heads_kv;
+  p.dim = dim;
+  p.page_size = page_size;
+  p.group = heads / heads_kv;
+  p.rows = q_len * p.group;
+  p.n_pages = n_phys_tokens / page_size;
+  p.softcap = softcap;
+  if (softcap > 0.f) {
+    p.score_scale = sm_scale;
+    p.cap_log2e = softcap * kLog2e;
+    p.inv_cap_scale = sm_scale / softcap;
+  } else {
+    p.score_scale = sm_scale * kLog2e;
+  }
+  p.causal = causal ? 1 : 0;
+  p.max_splits = plan.max_splits;
+  p.split_tokens = plan.split_tokens;
+  p.n_parts = plan.n_parts;
+
+  hipStream_t s = (hipStream_t)hip_stream;
+  const char* err;
+  if (plan.kernel == MI355_KERNEL_GENERIC) {
+    err = launch_generic(p, q_dtype, kv_dtype, s);
+    if (!err) err = launch_generic_combine(p, q_dtype, s);
+  } else {
+    err = launch_mfma(p, q_dtype, kv_dtype, s);
+  }
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  return MI355_OK;
+}
+
+int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
+                       void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size, int64_t n_phys_tokens,
+                       void* hip_stream) {
+  if (batch < 0 || max_len < 0) return fail(MI355_EINVAL, "batch and max_len must be non-negative");
+  if (batch > 65535) return fail(MI355_EUNSUPPORTED, "batch %d exceeds 65535", batch);
+  if (page_size <= 0) return fail(MI355_EINVAL, "page_size must be positive");
+  if (row_bytes <= 0 || row_bytes % 4 != 0) return fail(MI355_EINVAL, "row_bytes must be a positive multiple of 4");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens must be a positive multiple of page_size");
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (batch == 0 || max_len == 0) return MI355_OK;
+  if (!cache || !seqlens || !block_table || !dense_out) return fail(MI355_EINVAL, "null pointer argument");
+  const char* err = launch_gather_probe(cache, seqlens, block_table, bt_row_stride, dense_out, batch, max_len, row_bytes,
+                                        page_size, n_phys_tokens / page_size, (hipStream_t)hip_stream);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  return MI355_OK;
+}
+
+int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int32_t* seqlens, const int32_t* block_table,
+                        int64_t bt_row_stride, int batch, int heads_kv, int dim, int page_size, int64_t n_phys_tokens,
+                        int x_dtype, void* hip_stream) {
+  if (batch < 0 || batch > 65535) return fail(MI355_EINVAL, "batch must be in [0, 65535]");
+  if (heads_kv <= 0) return fail(MI355_EINVAL, "heads_kv must be positive");
+  if (dim != 64 && dim != 128 && dim != 256) return fail(MI355_EUNSUPPORTED, "head dim %d is not served (64, 128 or 256)", dim);
+  if (page_size <= 0) return fail(MI355_EINVAL, "page_size must be positive");
+  if (!is_q_dtype(x_dtype)) return fail(MI355_EINVAL, "x_dtype must be bf16 or fp16");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens must be a positive multiple of page_size");
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (batch == 0) return MI355_OK;
+  if (!x_new || !cache || !scale || !seqlens || !block_table) return fail(MI355_EINVAL, "null pointer argument");
+  const char* err = launch_kv_append_fp8(x_new, cache, scale, seqlens, block_table, bt_row_stride, batch, heads_kv, dim,
+                                         page_size, n_phys_tokens / page_size, x_dtype, (hipStream_t)hip_stream);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  return MI355_OK;
+}
+
+}  // extern "C"

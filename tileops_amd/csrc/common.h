@@ -1,0 +1,71 @@
+// Shared host/device declarations for the gfx950 paged GQA decode library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355_tileops.h"
+
+namespace mi355 {
+
+constexpr float kLog2e = 1.4426950408889634f;
+// Finite stand-in for "-infinity" as the running maximum: exp2(-inf - kNegFloor) == 0 and
+// exp2(kNegFloor - kNegFloor) == 1, so empty tiles and empty splits never produce NaN.
+constexpr float kNegFloor = -1.0e30f;
+
+// Everything one decode call needs, passed to the kernels by value.
+struct DecodeParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* k_scale;
+  const float* v_scale;
+  const int32_t* seqlens;
+  const int32_t* block_table;
+  int64_t bt_row_stride;
+  void* out;
+  float* part_o;    // workspace: normalised partial outputs, fp32
+  float* part_lse;  // workspace: log2-domain log-sum-exp per partial (-inf = empty)
+  int batch, q_len, heads, heads_kv, dim, page_size;
+  int group;        // heads / heads_kv
+  int rows;         // q_len * group : query rows that share one kv head
+  int64_t n_pages;  // n_phys_tokens / page_size
+  float score_scale;  // sm_scale (softcap on) or sm_scale * log2e (softcap off)
+  float softcap;      // 0 = off
+  float cap_log2e;    // softcap * log2e
+  float inv_cap_scale;  // sm_scale / softcap
+  int causal;
+  // generic kernel: fixed-length KV splits per sequence
+  int max_splits;
+  int split_tokens;
+  // MFMA kernel: even partition of the KV tile stream
+  int n_parts;
+};
+
+// Number of KV splits of one sequence and the (tile-aligned) tokens per split, generic kernel.
+// Used identically by the attention kernel and its combine kernel.
+__host__ __device__ inline void split_geometry(int len, int split_tokens, int max_splits, int* n_splits, int* chunk) {
+  int n = (len + split_tokens - 1) / split_tokens;
+  if (n > max_splits) n = max_splits;
+  if (n < 1) n = 1;
+  int c = (len + n - 1) / n;
+  c = (c + 63) / 64 * 64;
+  if (c < 64) c = 64;
+  *chunk = c;
+  *n_splits = len > 0 ? (len + c - 1) / c : 1;
+}
+
+// --- launchers (defined in the kernel translation units) -----------------------------------------
+const char* launch_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
+const char* launch_generic_combine(const DecodeParams& p, int q_dtype, hipStream_t s);
+bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap);
+int mfma_num_parts(int heads_kv, int rows, int kv_dtype);
+size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim);
+const char* launch_mfma(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
+const char* launch_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
+                                void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size,
+                                int64_t n_pages, hipStream_t s);
+const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, const int32_t* seqlens,
+                                 const int32_t* block_table, int64_t bt_row_stride, int batch, int heads_kv, int dim,
+                                 int page_size, int64_t n_pages, int x_dtype, hipStream_t s);
+
+}  // namespace mi355

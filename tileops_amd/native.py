@@ -1,0 +1,191 @@
+"""ctypes binding of ``libmi355_tileops.so`` (the C ABI declared in ``include/mi355_tileops.h``).
+
+torch is used here only for device memory and streams: tensors are handed over as raw ``data_ptr()``
+values plus the current HIP stream.  There is no CPU or eager-torch fallback: if the library is missing
+or the device is not a gfx950 GPU, calls raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_tileops.so"
+ABI_VERSION = 1
+
+DT_BF16, DT_FP16, DT_FP8_E4M3FN = 0, 1, 2
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+KERNEL_NAMES = {KERNEL_AUTO: "auto", KERNEL_GENERIC: "generic", KERNEL_MFMA: "mfma"}
+
+EXPORTED_SYMBOLS = (
+    "mi355_abi_version",
+    "mi355_last_error",
+    "mi355_gqa_paged_decode_workspace",
+    "mi355_gqa_paged_decode",
+    "mi355_gather_probe",
+    "mi355_kv_append_fp8",
+)
+
+
+class NativeLibraryError(RuntimeError):
+    """The HIP library is missing, stale, or reported an error."""
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+
+_c_int, _c_i64, _c_f32, _c_vp, _c_sz = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    lib.mi355_abi_version.restype = _c_int
+    lib.mi355_abi_version.argtypes = []
+    lib.mi355_last_error.restype = ctypes.c_char_p
+    lib.mi355_last_error.argtypes = []
+    lib.mi355_gqa_paged_decode_workspace.restype = _c_int
+    lib.mi355_gqa_paged_decode_workspace.argtypes = [
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int,
+        ctypes.POINTER(_c_sz), ctypes.POINTER(_c_int), ctypes.POINTER(_c_int),
+    ]
+    lib.mi355_gqa_paged_decode.restype = _c_int
+    lib.mi355_gqa_paged_decode.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
+        _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
+    ]
+    lib.mi355_gather_probe.restype = _c_int
+    lib.mi355_gather_probe.argtypes = [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_int, _c_i64, _c_i64, _c_int, _c_i64, _c_vp]
+    lib.mi355_kv_append_fp8.restype = _c_int
+    lib.mi355_kv_append_fp8.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_vp,
+    ]
+
+
+def load() -> ctypes.CDLL:
+    """Load the in-tree shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise NativeLibraryError(
+                f"{LIB_PATH} is missing: build it with `python -m tileops_amd.build` "
+                "(there is no CPU fallback for the MI355X kernels)"
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for sym in EXPORTED_SYMBOLS:
+            if not hasattr(lib, sym):
+                raise NativeLibraryError(f"{LIB_PATH} does not export {sym}")
+        _declare(lib)
+        got = lib.mi355_abi_version()
+        if got != ABI_VERSION:
+            raise NativeLibraryError(f"{LIB_PATH} has ABI version {got}, this package expects {ABI_VERSION}; rebuild")
+        _lib = lib
+        return lib
+
+
+def last_error() -> str:
+    return load().mi355_last_error().decode("utf-8", "replace")
+
+
+def _check(rc: int) -> None:
+    if rc == 0:
+        return
+    msg = last_error()
+    if rc in (-1,):
+        raise ValueError(msg)
+    if rc == -2:
+        raise NotImplementedError(msg)
+    raise NativeLibraryError(f"mi355 error {rc}: {msg}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return DT_BF16
+    if dtype == torch.float16:
+        return DT_FP16
+    if dtype == torch.float8_e4m3fn:
+        return DT_FP8_E4M3FN
+    raise ValueError(f"dtype {dtype} has no MI355X kernel (bfloat16, float16, float8_e4m3fn)")
+
+
+def is_gfx950(device: torch.device) -> bool:
+    """True iff *device* is a ROCm GPU whose architecture is gfx950 (MI350X / MI355X)."""
+    if device.type != "cuda" or torch.version.hip is None or not torch.cuda.is_available():
+        return False
+    name = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
+    return name.split(":")[0] == "gfx950"
+
+
+def require_gfx950(device: torch.device) -> None:
+    if not is_gfx950(device):
+        raise NativeLibraryError(f"device {device} is not a gfx950 (MI355X) GPU; these kernels run nowhere else")
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def decode_workspace(
+    batch: int, q_len: int, heads: int, heads_kv: int, dim: int, page_size: int, max_blocks_per_seq: int,
+    q_dtype: torch.dtype, kv_dtype: torch.dtype, num_split: int = 0, kernel: int = KERNEL_AUTO,
+) -> tuple[int, int, int]:
+    """(workspace_bytes, num_split, kernel) for a decode call of this shape.  Touches no device."""
+    lib = load()
+    nbytes, nsplit, kout = _c_sz(0), _c_int(0), _c_int(0)
+    _check(lib.mi355_gqa_paged_decode_workspace(
+        batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, dtype_code(q_dtype), dtype_code(kv_dtype),
+        num_split, kernel, ctypes.byref(nbytes), ctypes.byref(nsplit), ctypes.byref(kout)))
+    return int(nbytes.value), int(nsplit.value), int(kout.value)
+
+
+def paged_decode(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
+    seqlens: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, workspace: Optional[torch.Tensor], *,
+    batch: int, q_len: int, heads: int, heads_kv: int, dim: int, page_size: int,
+    sm_scale: float, softcap: float, causal: bool, num_split: int, kernel: int,
+) -> None:
+    """Enqueue one decode call on the current stream of ``q.device``.  Arguments are assumed validated."""
+    lib = load()
+    _check(lib.mi355_gqa_paged_decode(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0), out.data_ptr(),
+        workspace.data_ptr() if workspace is not None else None,
+        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        batch, q_len, heads, heads_kv, dim, page_size, k.shape[0],
+        dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
+        int(num_split), int(kernel), _stream_ptr(q.device)))
+
+
+def gather_probe(cache: torch.Tensor, seqlens: torch.Tensor, block_table: torch.Tensor, page_size: int, max_len: int) -> torch.Tensor:
+    """Dense ``[batch, max_len, *cache.shape[1:]]`` copy of the rows a decode call would read
+    (rows past each sequence's length are zero).  Device page arithmetic only -- the index-probe."""
+    require_gfx950(cache.device)
+    lib = load()
+    batch = seqlens.shape[0]
+    row_bytes = cache[0].numel() * cache.element_size()
+    out = torch.zeros((batch, max_len) + tuple(cache.shape[1:]), dtype=cache.dtype, device=cache.device)
+    _check(lib.mi355_gather_probe(
+        cache.data_ptr(), seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0), out.data_ptr(),
+        batch, max_len, row_bytes, page_size, cache.shape[0], _stream_ptr(cache.device)))
+    return out
+
+
+def kv_append_fp8(x_new: torch.Tensor, cache: torch.Tensor, scale: torch.Tensor, seqlens: torch.Tensor,
+                  block_table: torch.Tensor, page_size: int) -> None:
+    """Quantize ``x_new [batch, heads_kv, dim]`` per (token, head) and store it at each sequence's last position."""
+    require_gfx950(cache.device)
+    lib = load()
+    batch, heads_kv, dim = x_new.shape
+    _check(lib.mi355_kv_append_fp8(
+        x_new.data_ptr(), cache.data_ptr(), scale.data_ptr(), seqlens.data_ptr(), block_table.data_ptr(),
+        block_table.stride(0), batch, heads_kv, dim, page_size, cache.shape[0], dtype_code(x_new.dtype),
+        _stream_ptr(cache.device)))
