@@ -40,7 +40,9 @@ uint8_t fp8_e4m3fn_encode(float x) {
   uint8_t sign = (uint8_t)((bits >> 24) & 0x80);
   float a = fabsf(x);
   if (!(a == a)) return sign | 0x7F;          /* NaN */
-  if (a >= 464.0f) return sign | 0x7F;        /* 464 is the midpoint between 448 and the missing 480 */
+  if (isinf(a)) return sign | 0x7F;
+  /* 464 is the midpoint between 448 (even mantissa) and the NaN slot at 480: the tie itself rounds to 448,
+   * anything above it rounds into the NaN slot; both fall out of the general path below. */
   if (a < ldexpf(1.0f, -10)) return sign;     /* below half of the smallest subnormal (2^-9) -> 0 ; tie at 2^-10 -> even (0) */
   int e;
   (void)frexpf(a, &e);                        /* a = f * 2^e, f in [0.5,1) -> unbiased exponent e-1 */

@@ -1,0 +1,410 @@
+"""GPU parity tests of the paged GQA decode ops against the CPU oracle, through the op layer and the C ABI.
+
+The first block restates the reference's own test file case by case
+(tests/ops/attention/test_gqa_decode_paged.py:75-272): same shapes, same workload generator semantics, same
+comparison (max |diff| < 1e-3 and per-sequence cosine > 0.99 in fp16).  The rest covers what the reference
+leaves untested or does not have: bf16 numerics, ragged lengths and tails, permuted tables, NaN poison in
+unaddressed tokens, FP8 KV, multi-token causal queries, split invariance and the index-probe gather.
+Tolerances: atol = rtol = 2e-2 for bf16, 3e-2 for FP8 KV.
+"""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle.paged_gqa_decode_ref import quantize_kv_per_token, ref_paged_gqa_decode
+from tests.conftest import require_gfx950
+from tileops_amd import native
+from tileops_amd.ops import (
+    GroupedQueryAttentionDecodePagedWithKVCacheFwdOp as PagedOp,
+    GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp as MultiOp,
+)
+from tileops_amd.workloads import GroupedQueryAttentionDecodePagedWorkload
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+KERNELS = ["gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel"]
+
+
+def _maxdiff_cosine_compare(out, ref, batch, atol=1e-3):
+    """tests/ops/attention/test_gqa_decode_paged.py:17-28."""
+    out, ref = out.float().cpu(), ref.float()
+    max_diff = (out - ref).abs().max().item()
+    assert max_diff < atol, f"max diff {max_diff} too large (atol={atol})"
+    cos = F.cosine_similarity(out.reshape(batch, -1), ref.reshape(batch, -1), dim=-1, eps=1e-8)
+    assert cos.min() > 0.99, f"cosine similarity {cos.min().item()} too low"
+
+
+def _check_reference_style(op, wl, inputs, atol=1e-3):
+    q, k, v, lens, table = inputs
+    ref = ref_paged_gqa_decode(q.cpu(), k.cpu(), v.cpu(), lens.cpu(), table.cpu(), page_size=wl.page_size,
+                               sm_scale=wl.sm_scale, softcap=wl.softcap)
+    out = op(q, k, v, lens, table)
+    assert out.shape == q.shape and out.dtype == q.dtype
+    _maxdiff_cosine_compare(out, ref, wl.batch, atol)
+
+
+# --- the reference's cases ----------------------------------------------------------------------------------
+@pytest.mark.parametrize(
+    "batch, heads, heads_kv, seqlen_kv, dim, page_size",
+    [(1, 16, 8, 512, 128, 128), (2, 8, 4, 1024, 64, 256), (1, 32, 8, 256, 128, 64), (1, 8, 4, 1024, 64, 256),
+     (2, 16, 8, 512, 128, 128), (1, 16, 4, 2048, 128, 512), (1, 32, 16, 512, 64, 128)],
+)
+def test_gqa_decode_paged_op(batch, heads, heads_kv, seqlen_kv, dim, page_size):
+    require_gfx950()
+    wl = GroupedQueryAttentionDecodePagedWorkload(batch, heads, heads_kv, seqlen_kv, dim, page_size, torch.float16)
+    op = PagedOp(batch=batch, heads=heads, heads_kv=heads_kv, seqlen_kv=seqlen_kv, dim=dim, page_size=page_size, tune=False)
+    _check_reference_style(op, wl, wl.gen_inputs(DEV))
+
+
+def test_gqa_decode_paged_non_divisible_128_page_split():
+    """page_size=192 uses 64-token tiles without skipping page tails; reversed block table, full length."""
+    require_gfx950()
+    batch, heads, heads_kv, seqlen_kv, dim, page_size = 1, 16, 4, 3072, 128, 192
+    wl = GroupedQueryAttentionDecodePagedWorkload(batch, heads, heads_kv, seqlen_kv, dim, page_size, torch.float16)
+    q, k, v, lens, table = wl.gen_inputs(DEV)
+    lens.fill_(seqlen_kv)
+    table.copy_(torch.arange(seqlen_kv // page_size, device=DEV, dtype=torch.int32).flip(0).unsqueeze(0))
+    op = PagedOp(batch, heads, heads_kv, seqlen_kv, dim, page_size)
+    kernel = op._get_kernel((q,), torch.float16)
+    assert page_size % kernel.config["block_N"] == 0
+    assert {c["block_N"] for c in kernel.autotune_configs} == {64}
+    _check_reference_style(op, wl, (q, k, v, lens, table))
+
+
+@pytest.mark.parametrize("page_size", [96, 160, 224])
+def test_gqa_decode_paged_rejects_unsupported_page_tile(page_size):
+    require_gfx950()
+    op = PagedOp(1, 16, 4, page_size * 16, 128, page_size)
+    with pytest.raises(ValueError, match="matches no supported block_N"):
+        op._get_kernel((torch.empty(1, device=DEV),), torch.float16)
+
+
+@pytest.mark.parametrize("sm_scale, softcap", [pytest.param(0.25, None, id="custom-sm-scale"), pytest.param(None, 2.0, id="softcap")])
+def test_gqa_decode_paged_op_softmax_controls(sm_scale, softcap):
+    require_gfx950()
+    batch, heads, heads_kv, seqlen_kv, dim, page_size = 1, 16, 8, 512, 128, 128
+    wl = GroupedQueryAttentionDecodePagedWorkload(batch, heads, heads_kv, seqlen_kv, dim, page_size, torch.float16,
+                                                  sm_scale=sm_scale, softcap=softcap)
+    op = PagedOp(batch=batch, heads=heads, heads_kv=heads_kv, seqlen_kv=seqlen_kv, dim=dim, page_size=page_size,
+                 sm_scale=sm_scale, softcap=softcap)
+    _check_reference_style(op, wl, wl.gen_inputs(DEV))
+
+
+@pytest.mark.parametrize("real_len, reverse_pages", [pytest.param(512, False, id="no-split"), pytest.param(4096, True, id="ctx-reversed-pages")])
+def test_gqa_decode_paged_bs1_both_tiers(real_len, reverse_pages):
+    """Batch-1 short (one partial) and long (many partials) contexts, with output-distinguishing page translation."""
+    require_gfx950()
+    batch, heads, heads_kv, seqlen_kv, dim, page_size = 1, 32, 4, 4096, 128, 256
+    wl = GroupedQueryAttentionDecodePagedWorkload(batch, heads, heads_kv, seqlen_kv, dim, page_size, torch.float16)
+    op = PagedOp(batch, heads, heads_kv, seqlen_kv, dim, page_size)
+    q, k, v, lens, table = wl.gen_inputs(DEV, seed=0)
+    lens.fill_(real_len)
+    if reverse_pages:
+        table = table.flip(-1).contiguous()
+    _check_reference_style(op, wl, (q, k, v, lens, table))
+
+
+@pytest.mark.parametrize(
+    "batch, dtype, dim, page_size, softcap",
+    [pytest.param(2, torch.float16, 128, 256, None, id="batched"), pytest.param(1, torch.bfloat16, 128, 256, None, id="bf16"),
+     pytest.param(1, torch.float16, 64, 256, None, id="head-dim"), pytest.param(1, torch.float16, 128, 16, None, id="small-page"),
+     pytest.param(1, torch.float16, 128, 192, None, id="generic-page-tile"), pytest.param(1, torch.float16, 128, 256, 2.0, id="softcap")],
+)
+def test_gqa_decode_paged_dispatch_lands_on_a_kernel_that_serves_the_call(batch, dtype, dim, page_size, softcap):
+    """Every shape of the reference's dispatch table is served: by the specialised kernel inside its region,
+    by the general one elsewhere (head_dim 64 is outside the MFMA region)."""
+    require_gfx950()
+    seqlen_kv = 8064 if page_size == 192 else 8192
+    op = PagedOp(batch, 32, 4, seqlen_kv, dim, page_size, softcap=softcap)
+    kernel = op._get_kernel((torch.empty(1, device=DEV),), dtype)
+    call = op.attention_call(dtype, None, torch.device(DEV, 0))
+    expected = "GQADecodePagedMfmaKernel" if op.kernel_map["gqa_decode_paged_mfma_kernel"].applies(call) else "GQADecodePagedKernel"
+    assert kernel.__class__.__name__ == expected
+    if dim == 64:
+        assert expected == "GQADecodePagedKernel"
+
+
+# --- beyond the reference's coverage ------------------------------------------------------------------------
+def _ragged_case(B, H, H_kv, D, page, lens, dtype, q_len=1, fp8=False, seed=0, spare_pages=3, poison=True):
+    g = torch.Generator().manual_seed(seed)
+    need = [math.ceil(n / page) for n in lens]
+    n_pages = sum(need) + spare_pages
+    q_shape = (B, H, D) if q_len == 1 else (B, q_len, H, D)
+    q = torch.randn(q_shape, generator=g).to(dtype)
+    k = torch.randn(n_pages * page, H_kv, D, generator=g)
+    v = torch.randn(n_pages * page, H_kv, D, generator=g)
+    perm = torch.randperm(n_pages, generator=g)
+    table = torch.full((B, max(1, max(need))), int(perm[-1]), dtype=torch.int32)  # unused entries name a spare page
+    used = torch.zeros(n_pages * page, dtype=torch.bool)
+    at = 0
+    for b, n in enumerate(lens):
+        table[b, :need[b]] = perm[at:at + need[b]].to(torch.int32)
+        for j in range(need[b]):
+            p = int(perm[at + j])
+            used[p * page: p * page + min(page, n - j * page)] = True
+        at += need[b]
+    if fp8:
+        k, ks = quantize_kv_per_token(k)
+        v, vs = quantize_kv_per_token(v)
+    else:
+        k, v, ks, vs = k.to(dtype), v.to(dtype), None, None
+    if poison:  # every token no (table, length) pair addresses holds NaN; fp8 NaN is 0x7F
+        if fp8:
+            k.view(torch.uint8)[~used] = 0x7F
+            v.view(torch.uint8)[~used] = 0x7F
+            ks[~used] = float("nan")
+            vs[~used] = float("nan")
+        else:
+            k[~used] = float("nan")
+            v[~used] = float("nan")
+    return q, k, v, torch.tensor(lens, dtype=torch.int32), table, ks, vs
+
+
+def _run_and_compare(op, case, page, tol, **ref_kw):
+    q, k, v, lens, table, ks, vs = case
+    ref = ref_paged_gqa_decode(q, k, v, lens, table, page_size=page, k_scale=ks, v_scale=vs, **ref_kw)
+    dev = [None if t is None else t.to(DEV) for t in case]
+    out = op(*dev[:5]) if ks is None else op(*dev)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=tol, rtol=tol)
+    return out
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("dtype, fp8, tol", [(torch.bfloat16, False, 2e-2), (torch.float16, False, 2e-2), (torch.bfloat16, True, 3e-2)])
+def test_ragged_lengths_tails_permuted_tables_and_poison(kernel_key, dtype, fp8, tol):
+    """Lengths that are not page or tile multiples, a length-1 and a length-0 sequence, a far longer neighbour
+    (empty splits for the short ones), every sequence on its own permuted pages, NaN everywhere else."""
+    require_gfx950()
+    lens = [1, 0, 63, 64, 65, 777, 4099, 130]
+    case = _ragged_case(len(lens), 32, 8, 128, 64, lens, dtype, fp8=fp8, seed=21)
+    op = PagedOp(len(lens), 32, 8, case[1].shape[0], 128, 64)
+    if not _serves(op, kernel_key, dtype, fp8):
+        pytest.skip(f"{kernel_key} does not serve this shape")
+    _force(op, kernel_key)
+    _run_and_compare(op, case, 64, tol)
+
+
+def _serves(op, key, dtype, fp8):
+    call = op.attention_call(dtype, torch.float8_e4m3fn if fp8 else None, torch.device(DEV, 0))
+    return op.kernel_map[key].refusal(call) is None
+
+
+def _force(op, key):
+    """Make selection return *key* (the other key is removed from the map)."""
+    op.kernel_map = {key: op.kernel_map[key]}
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("page", [16, 32, 64, 128, 256])
+def test_page_sizes(kernel_key, page):
+    require_gfx950()
+    lens = [300, 1000, 17]
+    case = _ragged_case(3, 32, 8, 128, page, lens, torch.bfloat16, seed=22)
+    op = PagedOp(3, 32, 8, case[1].shape[0], 128, page)
+    if not _serves(op, kernel_key, torch.bfloat16, False):
+        pytest.skip(f"{kernel_key} does not serve page_size {page}")
+    _force(op, kernel_key)
+    _run_and_compare(op, case, page, 2e-2)
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("heads, heads_kv", [(8, 8), (16, 8), (64, 8), (128, 8), (4, 1), (24, 3)])
+def test_group_sizes(kernel_key, heads, heads_kv):
+    require_gfx950()
+    lens = [200, 1500]
+    case = _ragged_case(2, heads, heads_kv, 128, 64, lens, torch.bfloat16, seed=23)
+    op = PagedOp(2, heads, heads_kv, case[1].shape[0], 128, 64)
+    if not _serves(op, kernel_key, torch.bfloat16, False):
+        pytest.skip(f"{kernel_key} does not serve heads {heads}/{heads_kv}")
+    _force(op, kernel_key)
+    _run_and_compare(op, case, 64, 2e-2)
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("q_len, is_causal", [(8, True), (3, True), (4, False)])
+def test_multi_token_causal_chunk(kernel_key, fp8, q_len, is_causal):
+    require_gfx950()
+    lens = [1500, 300, q_len, 65]
+    case = _ragged_case(4, 64, 8, 128, 64, lens, torch.bfloat16, q_len=q_len, fp8=fp8, seed=24)
+    op = MultiOp(4, q_len, 64, 8, case[1].shape[0], 128, 64, is_causal=is_causal)
+    if not _serves(op, kernel_key, torch.bfloat16, fp8):
+        pytest.skip(f"{kernel_key} does not serve q_len {q_len}")
+    _force(op, kernel_key)
+    out = _run_and_compare(op, case, 64, 3e-2 if fp8 else 2e-2, is_causal=is_causal)
+    if is_causal:
+        # query i of the chunk equals a single-token decode at length len - q_len + i + 1
+        q, k, v, lens_t, table, ks, vs = [None if t is None else t.to(DEV) for t in case]
+        single = PagedOp(4, 64, 8, k.shape[0], 128, 64)
+        i = q_len - 2
+        lens_i = (lens_t - q_len + i + 1).clamp(min=0).to(torch.int32)
+        args = (q[:, i].contiguous(), k, v, lens_i, table) + (() if ks is None else (ks, vs))
+        torch.testing.assert_close(out[:, i].float(), single(*args).float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("softcap", [0.0, 30.0])
+def test_closed_forms_on_device(softcap):
+    require_gfx950()
+    lens = [100, 1, 700]
+    q, k, v, lens_t, table, _, _ = _ragged_case(3, 32, 8, 128, 64, lens, torch.bfloat16, seed=25)
+    op = PagedOp(3, 32, 8, k.shape[0], 128, 64, softcap=softcap or None)
+    dev = [t.to(DEV) for t in (q, k, v, lens_t, table)]
+    out0 = op(torch.zeros_like(dev[0]), *dev[1:]).float().cpu()     # q = 0 -> mean of V over the valid tokens
+    for b, n in enumerate(lens):
+        pages = table[b, : math.ceil(n / 64)].long()
+        rows = v.view(-1, 64, 8, 128)[pages].reshape(-1, 8, 128)[:n].float()
+        torch.testing.assert_close(out0[b], rows.mean(0).repeat_interleave(4, dim=0), atol=1e-2, rtol=1e-2)
+    out = op(*dev).float().cpu()
+    torch.testing.assert_close(out[1], v[int(table[1, 0]) * 64].float().repeat_interleave(4, dim=0), atol=1e-2, rtol=1e-2)  # len 1
+
+
+def test_generic_kernel_is_invariant_to_the_split_count():
+    require_gfx950()
+    lens = [4099, 777]
+    q, k, v, lens_t, table, _, _ = [None if t is None else t.to(DEV) for t in _ragged_case(2, 32, 8, 128, 64, lens, torch.bfloat16, seed=26)]
+    outs = []
+    for ns in (1, 2, 5, 64):
+        out = torch.empty_like(q)
+        nbytes, nsplit, _ = native.decode_workspace(2, 1, 32, 8, 128, 64, table.shape[1], q.dtype, k.dtype, ns, native.KERNEL_GENERIC)
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=DEV)
+        native.paged_decode(q, k, v, None, None, lens_t, table, out, ws, batch=2, q_len=1, heads=32, heads_kv=8, dim=128,
+                            page_size=64, sm_scale=128 ** -0.5, softcap=0.0, causal=True, num_split=nsplit, kernel=native.KERNEL_GENERIC)
+        outs.append(out.float())
+    for o in outs[1:]:
+        torch.testing.assert_close(o, outs[0], atol=8e-3, rtol=8e-3)  # fp32 partials: differences are bf16 output rounding
+
+
+def test_kernels_agree_with_each_other_and_joint_page_permutation_is_bit_invariant():
+    require_gfx950()
+    lens = [2000, 513, 64]
+    case = _ragged_case(3, 32, 8, 128, 64, lens, torch.bfloat16, seed=27, poison=False)
+    q, k, v, lens_t, table, _, _ = [None if t is None else t.to(DEV) for t in case]
+    outs = {}
+    for key in KERNELS:
+        op = PagedOp(3, 32, 8, k.shape[0], 128, 64)
+        if not _serves(op, key, torch.bfloat16, False):
+            continue
+        _force(op, key)
+        outs[key] = op(q, k, v, lens_t, table)
+        # move every physical page and rename it in the table: the same rows are read, so not a bit may change
+        n_pages = k.shape[0] // 64
+        sigma = torch.randperm(n_pages, generator=torch.Generator().manual_seed(5)).to(DEV)
+        k2, v2 = torch.empty_like(k), torch.empty_like(v)
+        k2.view(n_pages, 64, 8, 128)[sigma] = k.view(n_pages, 64, 8, 128)
+        v2.view(n_pages, 64, 8, 128)[sigma] = v.view(n_pages, 64, 8, 128)
+        table2 = sigma[table.long()].to(torch.int32)
+        assert torch.equal(op(q, k2, v2, lens_t, table2), outs[key])
+    vals = list(outs.values())
+    for o in vals[1:]:
+        torch.testing.assert_close(o.float(), vals[0].float(), atol=2e-2, rtol=2e-2)
+
+
+def test_wide_block_table_like_the_reference_contract_and_strided_rows():
+    """The reference hands over block_table [B, N_kv/page] (pool-wide); only the leading ceil(len/page) entries matter."""
+    require_gfx950()
+    lens = [900, 100]
+    q, k, v, lens_t, table, _, _ = _ragged_case(2, 32, 8, 128, 64, lens, torch.bfloat16, seed=28)
+    n_pages = k.shape[0] // 64
+    wide = torch.full((2, n_pages), n_pages - 1, dtype=torch.int32)
+    wide[:, : table.shape[1]] = table
+    op = PagedOp(2, 32, 8, k.shape[0], 128, 64)
+    ref = ref_paged_gqa_decode(q, k, v, lens_t, table, page_size=64)
+    out = op(q.to(DEV), k.to(DEV), v.to(DEV), lens_t.to(DEV), wide.to(DEV))
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=2e-2, rtol=2e-2)
+    padded = torch.zeros(2, n_pages + 5, dtype=torch.int32, device=DEV)
+    padded[:, :n_pages] = wide.to(DEV)
+    out2 = op(q.to(DEV), k.to(DEV), v.to(DEV), lens_t.to(DEV), padded[:, :n_pages])  # row stride != width
+    assert torch.equal(out2, out)
+
+
+def test_gather_probe_is_bit_identical_to_torch_indexing():
+    """Index-probe: K[t, h, d] encodes the physical token t, so any page-arithmetic slip shows as a wrong id."""
+    require_gfx950()
+    page, H_kv, D = 64, 8, 128
+    lens = [1, 64, 65, 1000, 4097]
+    need = [math.ceil(n / page) for n in lens]
+    n_pages = sum(need) + 7
+    g = torch.Generator().manual_seed(31)
+    perm = torch.randperm(n_pages, generator=g)
+    table = torch.zeros(len(lens), max(need), dtype=torch.int32)
+    at = 0
+    for b, c in enumerate(need):
+        table[b, :c] = perm[at:at + c].to(torch.int32)
+        at += c
+    tok = torch.arange(n_pages * page, dtype=torch.int32)
+    probe = (tok[:, None, None] * 1024 + torch.arange(H_kv, dtype=torch.int32)[None, :, None] * 128
+             + torch.arange(D, dtype=torch.int32)[None, None, :]).contiguous()        # int32 rows: every element names itself
+    lens_t = torch.tensor(lens, dtype=torch.int32)
+    max_len = max(lens)
+    for cache in (probe, probe.view(torch.float32)):
+        dense = native.gather_probe(cache.to(DEV), lens_t.to(DEV), table.to(DEV), page, max_len).cpu()
+        for b, n in enumerate(lens):
+            want = cache.view(n_pages, page, H_kv, D)[table[b, : need[b]].long()].reshape(-1, H_kv, D)[:n]
+            assert torch.equal(dense[b, :n].view(torch.int32), want.view(torch.int32))
+            assert (dense[b, n:].view(torch.int32) == 0).all()
+    # byte-wide cache rows (fp8) and the [N_kv, H_kv] scale rows go through the same routine
+    k8 = torch.randint(0, 255, (n_pages * page, H_kv, D), dtype=torch.uint8, generator=g)
+    dense8 = native.gather_probe(k8.to(DEV), lens_t.to(DEV), table.to(DEV), page, max_len).cpu()
+    for b, n in enumerate(lens):
+        want = k8.view(n_pages, page, H_kv, D)[table[b, : need[b]].long()].reshape(-1, H_kv, D)[:n]
+        assert torch.equal(dense8[b, :n], want)
+
+
+def test_kv_append_fp8_matches_the_quantizer_bit_for_bit():
+    """Append-then-read: the appended row's bytes and scale equal the oracle quantizer's
+    (tests/ops/attention/test_gqa_prefill_paged.py:398-415 checks its fused append the same way)."""
+    require_gfx950()
+    page, H_kv, D, B = 64, 8, 128, 5
+    lens = [1, 64, 65, 200, 130]
+    case = _ragged_case(B, 32, H_kv, D, page, lens, torch.bfloat16, fp8=True, seed=33, poison=False)
+    q, k8, v8, lens_t, table, ks, vs = case
+    g = torch.Generator().manual_seed(34)
+    x_new = (torch.randn(B, H_kv, D, generator=g) * torch.tensor([1e-6, 0.1, 1.0, 10.0, 300.0])[:, None, None]).to(torch.bfloat16)
+    want_q, want_s = quantize_kv_per_token(x_new)
+    kd, sd = k8.to(DEV), ks.to(DEV)
+    before_k, before_s = kd.clone(), sd.clone()
+    native.kv_append_fp8(x_new.to(DEV), kd, sd, lens_t.to(DEV), table.to(DEV), page)
+    torch.cuda.synchronize()
+    touched = torch.zeros(k8.shape[0], dtype=torch.bool)
+    for b, n in enumerate(lens):
+        phys = int(table[b, (n - 1) // page]) * page + (n - 1) % page
+        touched[phys] = True
+        assert torch.equal(kd[phys].cpu().view(torch.uint8), want_q[b].view(torch.uint8))
+        assert torch.equal(sd[phys].cpu(), want_s[b])
+    assert torch.equal(kd.cpu().view(torch.uint8)[~touched], before_k.cpu().view(torch.uint8)[~touched])
+    assert torch.equal(sd.cpu()[~touched], before_s.cpu()[~touched])
+
+
+def test_external_builder_path_runs_the_same_kernels():
+    """The plug-in's build_kernel, reached through the seam, gives the same bits as the in-tree path."""
+    require_gfx950()
+    from tileops_amd import backend, tileops_plugin
+
+    saved = backend.snapshot()
+    try:
+        backend.restore(backend._State({}, {}, [], None))
+        tileops_plugin.register(into=backend)
+        case = _ragged_case(2, 32, 8, 128, 64, [700, 90], torch.bfloat16, seed=35)
+        dev = [t.to(DEV) for t in case[:5]]
+        ext = PagedOp(2, 32, 8, dev[1].shape[0], 128, 64)
+        out_ext = ext(*dev)
+        assert ext._settled_target == "mi355x"
+        builtin = PagedOp(2, 32, 8, dev[1].shape[0], 128, 64, target=backend.BUILTIN)
+        assert torch.equal(builtin(*dev), out_ext)
+    finally:
+        backend.restore(saved)
+
+
+def test_tune_picks_a_config_and_stays_correct():
+    require_gfx950()
+    wl = GroupedQueryAttentionDecodePagedWorkload(2, 32, 8, 4096, 128, 64, torch.float16)
+    op = PagedOp(2, 32, 8, 4096, 128, 64, tune=True)
+    inputs = wl.gen_inputs(DEV)
+    _check_reference_style(op, wl, inputs)
+    kernel = next(iter(op.built_kernels(next(iter(op._kernel_roles))).values()))
+    assert kernel.config in kernel.autotune_configs

@@ -1,0 +1,291 @@
+"""L1 host wrappers of the gfx950 HIP kernels.
+
+``Kernel`` reproduces the lifecycle of the reference's kernel base
+(src/tileops/kernels/kernel_base.py:47-365): architecture check at construction, ``config`` /
+``default_config`` / ``autotune_configs``, and the selection protocol ``applies`` / ``general`` /
+``refusal``.  The two concrete classes take the place of ``GQADecodePagedKernel``
+(src/tileops/kernels/attention/gqa_decode_paged.py:513-746) and of the specialised sibling
+(``GQADecodePagedBs1Kernel``, src/tileops/kernels/attention/gqa_decode_bs1_paged.py:177-299): the general
+VALU kernel serves every call, the MFMA kernel states the narrower region it serves and wins there.
+
+Nothing here computes attention: ``forward`` allocates the output and the workspace with torch and
+enqueues the HIP kernels through the C ABI.  No host read-back of device data happens on the call path.
+"""
+
+from __future__ import annotations
+
+import functools
+import itertools
+from dataclasses import dataclass
+from typing import Any, Optional
+
+import torch
+
+from . import native
+
+__all__ = [
+    "AttentionCall", "GQADecodePagedKernel", "GQADecodePagedMfmaKernel", "Kernel", "PAGED_DECODE_KEYS",
+    "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch",
+]
+
+#: Dispatch keys of the paged decode ops, in no particular order (selection never reads the order).
+PAGED_DECODE_KEYS = ("gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel")
+
+GFX950_ARCH = 95  # torch.cuda.get_device_capability() == (9, 5) on gfx950
+
+
+@functools.lru_cache(maxsize=None)
+def get_arch(device_index: Optional[int] = None) -> Optional[int]:
+    """major*10+minor of a ROCm device, or None when no GPU is visible."""
+    if not torch.cuda.is_available():
+        return None
+    major, minor = torch.cuda.get_device_capability(device_index)
+    return major * 10 + minor
+
+
+def _as_torch_dtype(dtype: Any) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        return dtype
+    return getattr(torch, str(dtype))
+
+
+@dataclass(frozen=True)
+class AttentionCall:
+    """Facts of one paged decode call that kernel selection filters on
+    (reference: src/tileops/kernels/attention/call_spec.py:44-76, kernels/call_spec.py:8-42)."""
+
+    dtype: torch.dtype
+    batch: int
+    heads: int
+    heads_kv: int
+    seqlen_kv: int
+    dim: int
+    page_size: int
+    sm_scale: float
+    softcap: float
+    tune: bool = False
+    kv_dtype: Optional[torch.dtype] = None
+    q_len: int = 1
+    is_causal: bool = True
+    arch: Optional[int] = None
+
+    @property
+    def group(self) -> int:
+        return self.heads // self.heads_kv
+
+
+def gqa_decode_paged_block_ns(page_size: int) -> tuple[int, ...]:
+    """KV tile heights that cover a page exactly, widest first.
+
+    Same rule and same messages as the reference (gqa_decode_paged.py:21-33): 128 or 64 when they divide
+    the page, the page itself below 64, otherwise the layout is rejected.
+    """
+    if page_size <= 0:
+        raise ValueError("page_size must be positive")
+    fits = tuple(n for n in (128, 64) if n <= page_size and page_size % n == 0)
+    if fits:
+        return fits
+    if page_size < 64:
+        return (page_size,)
+    raise ValueError(f"page_size={page_size} matches no supported block_N")
+
+
+def gqa_decode_paged_block_n(page_size: int) -> int:
+    return gqa_decode_paged_block_ns(page_size)[0]
+
+
+class Kernel:
+    """Base of the host-side kernel wrappers."""
+
+    supported_archs: Optional[list[int]] = None
+    #: True for the implementation that runs where no specialised one applies.
+    general: bool = False
+    autotune_configs: Optional[list[dict]] = None
+
+    def __init__(self, *, device_index: Optional[int] = None) -> None:
+        self.device_index = device_index
+        self._check_arch()
+        self.config: dict[str, Any] = {}
+
+    @classmethod
+    def applies(cls, call: Any) -> bool:
+        return True
+
+    @classmethod
+    def refusal(cls, call: Any) -> Optional[str]:
+        """Why this class cannot serve *call*, or None when it can."""
+        archs = cls.supported_archs
+        if archs is not None and call.arch not in archs:
+            return f"built for architectures {sorted(archs)}, device reports {call.arch}"
+        if not cls.applies(call):
+            return "does not serve this call"
+        return None
+
+    def _check_arch(self) -> None:
+        cls = type(self)
+        if cls.supported_archs is None:
+            return
+        arch = get_arch(self.device_index)
+        if arch not in cls.supported_archs:
+            where = "the current device" if self.device_index is None else f"cuda:{self.device_index}"
+            raise ValueError(
+                f"{cls.__name__} is built for architectures {sorted(cls.supported_archs)}, but {where} reports {arch}"
+            )
+
+    @property
+    def default_config(self) -> dict[str, Any]:
+        return {}
+
+    def init_config(self, config: Optional[dict[str, Any]] = None, tune: bool = False) -> None:
+        if tune and not self.autotune_configs:
+            tune = False
+        if tune:
+            self.autotune()
+        elif config is not None:
+            self.config = {k: (config[k] if config.get(k) is not None else v) for k, v in self.default_config.items()}
+        else:
+            self.config = dict(self.default_config)
+
+    def autotune(self) -> None:
+        raise NotImplementedError
+
+    def forward(self, *args: Any, **kwargs: Any) -> Any:
+        raise NotImplementedError
+
+    def __call__(self, *args: Any, **kwargs: Any) -> Any:
+        return self.forward(*args, **kwargs)
+
+
+class GQADecodePagedKernel(Kernel):
+    """General paged GQA decode on gfx950: the VALU HIP kernel plus fp32 split-KV combine.
+
+    Constructor arguments follow the reference class (gqa_decode_paged.py:526-538); ``groups`` is the
+    number of KV heads, as there.  ``kv_dtype`` (default: same as ``dtype``), ``q_len`` and ``is_causal``
+    are this package's extensions for an FP8 cache and multi-token queries.
+    """
+
+    supported_archs = [GFX950_ARCH]
+    general = True
+    _native_kernel = native.KERNEL_GENERIC
+
+    def __init__(self, batch: int, heads: int, groups: int, seqlen_kv: int, dim: int, page_size: int,
+                 dtype: Any = "float16", sm_scale: Optional[float] = None, softcap: float = 0.0,
+                 config: Optional[dict] = None, tune: bool = False, *, kv_dtype: Any = None, q_len: int = 1,
+                 is_causal: bool = True, device_index: Optional[int] = None) -> None:
+        super().__init__(device_index=device_index)
+        self.batch, self.heads, self.groups, self.seqlen_kv = batch, heads, groups, seqlen_kv
+        self.dim, self.page_size = dim, page_size
+        self.dtype = _as_torch_dtype(dtype)
+        self.kv_dtype = self.dtype if kv_dtype is None else _as_torch_dtype(kv_dtype)
+        self.q_len, self.is_causal = q_len, is_causal
+        self.sm_scale = dim ** -0.5 if sm_scale is None else sm_scale
+        self.softcap = softcap
+        self._supported_block_ns = gqa_decode_paged_block_ns(page_size)
+        if config is not None:
+            block_n = config.get("block_N")
+            if block_n is not None and block_n not in self._supported_block_ns:
+                raise ValueError(f"block_N={block_n} is not supported for page_size={page_size}")
+        if self.groups <= 0:
+            raise ValueError("groups must be positive")
+        if self.heads % self.groups != 0:
+            raise ValueError("heads must be divisible by groups")
+        if self.seqlen_kv <= 0:
+            raise ValueError("seqlen_kv must be positive")
+        if self.page_size <= 0:
+            raise ValueError("page_size must be positive")
+        if self.seqlen_kv % self.page_size != 0:
+            raise ValueError("seqlen_kv must be divisible by page_size")
+        self._plans: dict[tuple[int, int], tuple[int, int]] = {}
+        self.init_config(config, tune)
+
+    # -- config ----------------------------------------------------------------------------------------
+    @property
+    def default_config(self) -> dict[str, Any]:
+        # block_N is the page-contained tile the launch assumes; num_split 0 lets the library choose
+        return {"block_N": gqa_decode_paged_block_n(self.page_size), "num_split": 0}
+
+    @property
+    def autotune_configs(self) -> list[dict]:
+        return [{"block_N": n, "num_split": s} for n, s in itertools.product(self._supported_block_ns, (0, 8, 16, 32))]
+
+    def autotune(self) -> None:
+        """Time every ``autotune_configs`` entry on synthetic full-length inputs and keep the fastest."""
+        device = torch.device("cuda", self.device_index if self.device_index is not None else torch.cuda.current_device())
+        n_pages = self.seqlen_kv // self.page_size
+        q_shape = (self.batch, self.heads, self.dim) if self.q_len == 1 else (self.batch, self.q_len, self.heads, self.dim)
+        q = torch.randn(q_shape, device=device, dtype=self.dtype)
+        kv = torch.randn(2, self.seqlen_kv, self.groups, self.dim, device=device, dtype=torch.float32)
+        if self.kv_dtype == torch.float8_e4m3fn:
+            k, v = kv[0].clamp(-448, 448).to(self.kv_dtype), kv[1].clamp(-448, 448).to(self.kv_dtype)
+            ks = torch.full((self.seqlen_kv, self.groups), 0.01, device=device, dtype=torch.float32)
+            vs = ks.clone()
+        else:
+            k, v, ks, vs = kv[0].to(self.kv_dtype), kv[1].to(self.kv_dtype), None, None
+        lens = torch.full((self.batch,), self.seqlen_kv, dtype=torch.int32, device=device)
+        table = torch.arange(n_pages, dtype=torch.int32, device=device).unsqueeze(0).expand(self.batch, -1).contiguous()
+        best, best_ms = None, float("inf")
+        for cfg in self.autotune_configs:
+            self.config = dict(cfg)
+            for _ in range(3):
+                self.forward(q, k, v, lens, table, ks, vs)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(10):
+                self.forward(q, k, v, lens, table, ks, vs)
+            stop.record()
+            stop.synchronize()
+            ms = start.elapsed_time(stop) / 10
+            if ms < best_ms:
+                best, best_ms = dict(cfg), ms
+        self.config = best
+
+    # -- launch ----------------------------------------------------------------------------------------
+    def _plan(self, max_blocks_per_seq: int) -> tuple[int, int]:
+        key = (max_blocks_per_seq, int(self.config.get("num_split", 0)))
+        plan = self._plans.get(key)
+        if plan is None:
+            nbytes, nsplit, _ = native.decode_workspace(
+                self.batch, self.q_len, self.heads, self.groups, self.dim, self.page_size, max_blocks_per_seq,
+                self.dtype, self.kv_dtype, key[1], self._native_kernel)
+            plan = self._plans[key] = (nbytes, nsplit)
+        return plan
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor,
+                block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+                v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        native.require_gfx950(q.device)
+        nbytes, nsplit = self._plan(block_table.shape[1])
+        out = torch.empty_like(q)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
+        native.paged_decode(
+            q, k, v, k_scale, v_scale, real_seqlen_kv, block_table, out, workspace,
+            batch=self.batch, q_len=self.q_len, heads=self.heads, heads_kv=self.groups, dim=self.dim,
+            page_size=self.page_size, sm_scale=self.sm_scale, softcap=self.softcap, causal=self.is_causal,
+            num_split=nsplit, kernel=self._native_kernel)
+        return out
+
+
+class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
+    """MFMA paged GQA decode on gfx950: direct-to-LDS page gather, QK^T and PV on the matrix cores, the KV
+    tile stream partitioned evenly over all compute units.  Serves the region the HIP library reports as
+    supported (head_dim 128, page size a multiple of 16, ...); everything else stays on the general kernel."""
+
+    general = False
+    _native_kernel = native.KERNEL_MFMA
+
+    @classmethod
+    def applies(cls, call: AttentionCall) -> bool:
+        try:
+            native.decode_workspace(call.batch, call.q_len, call.heads, call.heads_kv, call.dim, call.page_size, 1,
+                                    call.dtype, call.kv_dtype or call.dtype, 0, native.KERNEL_MFMA)
+        except (NotImplementedError, ValueError):
+            return False
+        return True
+
+    @property
+    def default_config(self) -> dict[str, Any]:
+        return {"block_N": gqa_decode_paged_block_n(self.page_size), "num_split": 0}
+
+    @property
+    def autotune_configs(self) -> list[dict]:
+        return [dict(self.default_config)]

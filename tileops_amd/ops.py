@@ -1,0 +1,248 @@
+"""L2 ops: paged GQA decode over a KV page pool, bf16/fp16 or FP8-e4m3fn cache, on MI355X.
+
+``GroupedQueryAttentionDecodePagedWithKVCacheFwdOp`` keeps the reference op's contract
+(src/tileops/ops/attention/gqa.py:1357-1454): same constructor arguments, defaults and error messages
+(``_validate_gqa_dims`` :74-78, ``_validate_positive`` :66-71, scale/softcap defaults :81-90), same
+``forward(q, k, v, real_seqlen_kv, block_table)`` order, output = ``q``'s shape and dtype.  On top of it:
+
+* ``k``/``v`` may be ``float8_e4m3fn`` with trailing optional ``k_scale, v_scale [N_kv, H_kv]`` fp32
+  (dequant ``fp8.float() * scale``; scale rules follow the paged prefill op, gqa.py:992-999);
+* ``forward`` validates device, dtype, rank/shape, contiguity and metadata dtypes (the reference's forward
+  validates nothing; its sibling paged prefill op does, gqa.py:897-1046, and that is the template);
+* an external target's builder, once settled, is consulted *before* in-tree kernel selection, so a target
+  whose devices the in-tree kernels cannot run on is still reachable.
+
+``GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp`` is the multi-token (speculative-verify)
+sibling: ``q [B, S_q, H, D]``, the cache already holds the S_q new tokens, and the causal mask is
+bottom-right aligned (key j visible to query i iff ``j <= i + (len - S_q)``; gqa.py:558-562).
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .backend import Target
+from .kernels import PAGED_DECODE_KEYS, AttentionCall, GQADecodePagedKernel, GQADecodePagedMfmaKernel, get_arch
+from .op_base import _UNRESOLVED, Op
+
+__all__ = [
+    "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp",
+    "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp",
+]
+
+FP8 = torch.float8_e4m3fn
+
+
+def _validate_attention_dtype(dtype: torch.dtype) -> None:
+    if dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"Expected dtype torch.float16 or torch.bfloat16, got {dtype}")
+
+
+def _validate_positive(**values: int) -> None:
+    for name, value in values.items():
+        if value <= 0:
+            raise ValueError(f"{name} must be positive")
+
+
+def _validate_gqa_dims(heads: int, heads_kv: int, dim: int) -> None:
+    _validate_positive(heads=heads, heads_kv=heads_kv)
+    if heads % heads_kv != 0:
+        raise ValueError("heads must be divisible by heads_kv")
+    _validate_positive(dim=dim)
+
+
+def _attention_scale(dim: int, sm_scale: Optional[float]) -> float:
+    return dim ** -0.5 if sm_scale is None else sm_scale
+
+
+def _score_softcap(softcap: Optional[float]) -> float:
+    if softcap is None:
+        return 0.0
+    if softcap < 0:
+        raise ValueError("softcap must be non-negative")
+    return softcap
+
+
+class _PagedDecodeOp(Op):
+    """What the single-token op and its multi-token sibling share."""
+
+    q_len: int = 1
+    is_causal: bool = True
+    #: Set True to also check values that live on the device (scales finite and positive, block-table
+    #: entries inside the pool).  Costs a device read-back per call, so it is off on the serving path.
+    debug_checks: bool = False
+    _seen_call: Optional[dict] = None
+
+    def _init_common(self, batch: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int, page_size: int,
+                     sm_scale: Optional[float], softcap: Optional[float], kernel_map: Optional[Dict[str, type]],
+                     tune: bool, target: Target) -> None:
+        _validate_gqa_dims(heads, heads_kv, dim)
+        self.batch, self.heads, self.heads_kv, self.seqlen_kv, self.dim = batch, heads, heads_kv, seqlen_kv, dim
+        self.page_size = page_size
+        _validate_positive(page_size=page_size)
+        self.sm_scale = _attention_scale(dim, sm_scale)
+        self.softcap = _score_softcap(softcap)
+        self.tune = tune
+        if target is not None:
+            self.target = target
+        self.dispatch_kernel(kernel_map)
+
+    @property
+    def default_kernel_map(self) -> Dict[str, type]:
+        return {
+            "gqa_decode_paged_kernel": GQADecodePagedKernel,
+            "gqa_decode_paged_mfma_kernel": GQADecodePagedMfmaKernel,
+        }
+
+    def attention_call(self, dtype: torch.dtype, kv_dtype: Optional[torch.dtype] = None,
+                       device: Optional[torch.device] = None) -> AttentionCall:
+        """State what one call is, for selection to filter against.  Reads the device architecture (not the ctor)."""
+        index = device.index if device is not None and device.type == "cuda" else None
+        return AttentionCall(
+            dtype=dtype, kv_dtype=kv_dtype or dtype, batch=self.batch, heads=self.heads, heads_kv=self.heads_kv,
+            seqlen_kv=self.seqlen_kv, dim=self.dim, page_size=self.page_size, sm_scale=self.sm_scale,
+            softcap=self.softcap, tune=self.tune, q_len=self.q_len, is_causal=self.is_causal, arch=get_arch(index))
+
+    def _get_kernel(self, inputs: "tuple[torch.Tensor | None, ...]", dtype: torch.dtype,
+                    kv_dtype: Optional[torch.dtype] = None):
+        _validate_attention_dtype(dtype)
+        kv_dtype = kv_dtype or dtype
+        if self._builder is not None and self._builder is not _UNRESOLVED:
+            # an external target serves this instance: its builder chooses among its own kernels
+            return self.get_or_build_kernel("gqa_decode_paged_kernel", inputs)
+        device = next((t.device for t in inputs if t is not None), None)
+        call = self.attention_call(dtype, kv_dtype, device)
+        key = self.select_kernel_key(PAGED_DECODE_KEYS, call)
+
+        def build():
+            return self.kernel_map[key](
+                call.batch, call.heads, call.heads_kv, call.seqlen_kv, call.dim, call.page_size, call.dtype,
+                sm_scale=call.sm_scale, softcap=call.softcap, tune=call.tune, kv_dtype=call.kv_dtype,
+                q_len=call.q_len, is_causal=call.is_causal,
+                device_index=device.index if device is not None and device.type == "cuda" else None)
+
+        return self.get_or_build_kernel(key, inputs, key=(dtype, kv_dtype), build=build)
+
+    # -- validation ------------------------------------------------------------------------------------
+    def _q_shape(self) -> tuple[int, ...]:
+        return (self.batch, self.heads, self.dim) if self.q_len == 1 and not self._q_is_4d else (
+            self.batch, self.q_len, self.heads, self.dim)
+
+    _q_is_4d = False
+
+    def _validate_call(self, q, k, v, real_seqlen_kv, block_table, k_scale, v_scale) -> None:
+        named = {"q": q, "k": k, "v": v, "real_seqlen_kv": real_seqlen_kv, "block_table": block_table}
+        for name, t in named.items():
+            if not isinstance(t, torch.Tensor):
+                raise ValueError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+        self._validate_dtypes(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+        fp8 = k.dtype == FP8
+        if fp8 and (k_scale is None or v_scale is None):
+            raise ValueError("k_scale and v_scale are required when the KV cache is float8_e4m3fn")
+        if not fp8 and (k_scale is not None or v_scale is not None):
+            raise ValueError("k_scale and v_scale must be None unless the KV cache is float8_e4m3fn")
+        if fp8:
+            named.update(k_scale=k_scale, v_scale=v_scale)
+        for name, t in named.items():
+            if t.device != q.device:
+                raise ValueError(f"Expected {name} on {q.device}, got {t.device}")
+        want_q = self._q_shape()
+        if tuple(q.shape) != want_q:
+            raise ValueError(f"Expected q.shape {want_q}, got {tuple(q.shape)}")
+        want_kv = (self.seqlen_kv, self.heads_kv, self.dim)
+        for name, t in (("k", k), ("v", v)):
+            if tuple(t.shape) != want_kv:
+                raise ValueError(f"Expected {name}.shape {want_kv}, got {tuple(t.shape)}")
+        if tuple(real_seqlen_kv.shape) != (self.batch,):
+            raise ValueError(f"Expected real_seqlen_kv.shape {(self.batch,)}, got {tuple(real_seqlen_kv.shape)}")
+        if block_table.dim() != 2 or block_table.shape[0] != self.batch or block_table.shape[1] < 1:
+            raise ValueError(f"Expected block_table.shape ({self.batch}, num_pages), got {tuple(block_table.shape)}")
+        for name, t in (("q", q), ("k", k), ("v", v), ("real_seqlen_kv", real_seqlen_kv)):
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous")
+        if block_table.stride(1) != 1:
+            raise ValueError("block_table rows must be contiguous (stride(1) == 1)")
+        if fp8:
+            for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+                if tuple(t.shape) != (self.seqlen_kv, self.heads_kv):
+                    raise ValueError(f"Expected {name}.shape {(self.seqlen_kv, self.heads_kv)}, got {tuple(t.shape)}")
+                if not t.is_contiguous():
+                    raise ValueError(f"{name} must be contiguous")
+        if self.debug_checks:
+            if fp8:
+                for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+                    if not torch.all(torch.isfinite(t) & (t > 0)).item():
+                        raise ValueError(f"{name} must contain finite positive values")
+            if real_seqlen_kv.min().item() < 0:
+                raise ValueError("real_seqlen_kv must be non-negative")
+            need = (real_seqlen_kv.max().item() + self.page_size - 1) // self.page_size
+            if need > block_table.shape[1]:
+                raise ValueError(f"block_table has {block_table.shape[1]} columns but the longest sequence needs {need}")
+            if block_table.min().item() < 0 or block_table.max().item() >= self.seqlen_kv // self.page_size:
+                raise ValueError("block_table entries must lie in [0, seqlen_kv // page_size)")
+
+    def observe_call(self, real_seqlen_kv: torch.Tensor, kv_dtype: torch.dtype) -> None:
+        """Record the context lengths of a call so that ``eval_roofline`` prices the bytes actually addressed.
+        Reads device memory once; benchmarks call it outside the timed region."""
+        lens = real_seqlen_kv.to("cpu", torch.int64)
+        pages = (lens + self.page_size - 1) // self.page_size
+        self._seen_call = {
+            "sum_len": int(lens.sum()), "sum_pages": int(pages.sum()),
+            "kv_bytes": torch.empty((), dtype=kv_dtype).element_size(), "fp8": kv_dtype == FP8,
+        }
+
+    def _run(self, q, k, v, real_seqlen_kv, block_table, k_scale, v_scale) -> torch.Tensor:
+        self._validate_call(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+        self.dtype = q.dtype
+        inputs = (q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+        kernel = self._get_kernel(inputs, q.dtype, k.dtype)
+        if k_scale is None:
+            return kernel(q, k, v, real_seqlen_kv, block_table)
+        return kernel(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+
+
+class GroupedQueryAttentionDecodePagedWithKVCacheFwdOp(_PagedDecodeOp):
+    """Paged GQA decode with dynamic KV cache. Layout: Q [batch, heads, dim] (BHD);
+    K, V physical cache [seqlen_kv, heads_kv, dim]; real_seqlen_kv [batch]; block_table [batch, num_pages]."""
+
+    def __init__(self, batch: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int, page_size: int,
+                 sm_scale: Optional[float] = None, softcap: Optional[float] = None,
+                 kernel_map: Optional[Dict[str, type]] = None, tune: bool = False, *, target: Target = None) -> None:
+        self._init_common(batch, heads, heads_kv, seqlen_kv, dim, page_size, sm_scale, softcap, kernel_map, tune, target)
+
+    def _infer_output_shapes(self, q_shape, k_shape, v_shape, real_seqlen_kv_shape, block_table_shape,
+                             k_scale_shape=None, v_scale_shape=None) -> dict[str, tuple[int, ...]]:
+        """Manifest ``shape_rules``: ``o.shape == q.shape``."""
+        return {"o": tuple(q_shape)}
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor,
+                block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+                v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self._run(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+
+
+class GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp(_PagedDecodeOp):
+    """Multi-token paged GQA decode (speculative verify). Layout: Q [batch, q_len, heads, dim] (BSHD);
+    K, V physical cache [seqlen_kv, heads_kv, dim] already holding the q_len new tokens;
+    real_seqlen_kv [batch] counts them; block_table [batch, num_pages]."""
+
+    _q_is_4d = True
+
+    def __init__(self, batch: int, q_len: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int, page_size: int,
+                 is_causal: bool = True, sm_scale: Optional[float] = None, softcap: Optional[float] = None,
+                 kernel_map: Optional[Dict[str, type]] = None, tune: bool = False, *, target: Target = None) -> None:
+        _validate_positive(q_len=q_len)
+        self.q_len = q_len
+        self.is_causal = bool(is_causal)
+        self._init_common(batch, heads, heads_kv, seqlen_kv, dim, page_size, sm_scale, softcap, kernel_map, tune, target)
+
+    def _infer_output_shapes(self, q_shape, k_shape, v_shape, real_seqlen_kv_shape, block_table_shape,
+                             k_scale_shape=None, v_scale_shape=None) -> dict[str, tuple[int, ...]]:
+        return {"o": tuple(q_shape)}
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor,
+                block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+                v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self._run(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
