@@ -1,8 +1,663 @@
-// placeholder until the MFMA kernel lands
+// MFMA paged GQA decode for gfx950 (MI355X): head_dim 128, bf16/fp16 or FP8-e4m3fn KV.
+//
+// What it computes is the reference's split kernel + combine
+// (src/tileops/kernels/attention/gqa_decode_paged.py:209-374): per (sequence, kv head), online softmax in
+// the exp2 domain over the paged K/V rows, all query rows that share the kv head served from one read of
+// K/V; partial results merged by log-sum-exp weights.  How it is organised is specific to CDNA4:
+//
+//  * Work unit = one wave.  A wave owns (partition, kv head, block of query rows) and runs on its own: no
+//    workgroup barrier anywhere.  The KV "tile stream" (every 32-token tile of every sequence, in batch
+//    order) is cut into n_parts equal contiguous ranges computed on the device from real_seqlen_kv, so all
+//    compute units get the same number of tiles whatever the length distribution, and nothing is read back
+//    to the host.  A range that covers a whole sequence writes the output directly; a range that starts or
+//    ends inside a sequence writes an fp32 partial (at most two per wave) that the combine kernel merges.
+//  * Page gather = 128-bit direct-to-LDS loads (global_load_lds_dwordx4) with the non-temporal hint, 1 KiB
+//    per wave instruction covering whole 256-byte (bf16) or 128-byte (fp8) K/V rows, NS stages per wave in
+//    flight, waited on with s_waitcnt vmcnt.  The LDS image is XOR-swizzled by choosing which 16-byte chunk
+//    each lane fetches, so the reads below are bank-conflict free.
+//  * QK^T: S^T[token][row] = K . Q^T on v_mfma_f32_16x16x32 (K rows straight from LDS as the A operand,
+//    query rows resident in registers as B).  Having tokens on the M axis puts P in exactly the register
+//    layout the PV product needs as its B operand, so P never moves between lanes.
+//  * PV: O^T[d][row] += V^T . P^T, V^T fetched with LDS transpose reads (ds_read_b64_tr_b16 / _tr_b8).
+//    Query rows sit on the N axis = lane % 16, so every per-row softmax quantity (max, sum, rescale factor)
+//    is lane-local; the only cross-lane traffic is a two-step max/sum over the four 16-lane groups.
+//  * FP8: bytes are widened to bf16/fp16 on the LDS->register path (v_cvt_scalef32_pk_*_fp8, OCP e4m3fn);
+//    the per-token K scale multiplies the score and the V scale multiplies the probability, so no
+//    head_dim-wide multiplies are spent on dequantisation.  Scales ride the same direct-to-LDS pipeline.
 #include "common.h"
+#include "device_utils.h"
+
 namespace mi355 {
-bool mfma_supported(int, int, int, int, int, int, int, float) { return false; }
-int mfma_num_parts(int, int, int) { return 0; }
-size_t mfma_workspace_bytes(int, int, int, int) { return 0; }
-const char* launch_mfma(const DecodeParams&, int, int, hipStream_t) { return "MFMA kernel not built"; }
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
+
+constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
+constexpr int kD = 128;       // head dim served by this kernel
+constexpr int kNW = 4;        // waves per workgroup
+constexpr int kNumCU = 256;   // MI355X
+
+template <typename KVT> struct Geom {
+  static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
+  static constexpr int ROW = kD * ElemTraits<KVT>::bytes;  // bytes of one (token, kv head) row
+  static constexpr int TPI = 1024 / ROW;                   // tokens per direct-to-LDS instruction
+  static constexpr int NI = kCT / TPI;                     // instructions per K (or V) stage
+  static constexpr int KBYTES = kCT * ROW;
+  static constexpr int SCBYTES = FP8 ? 256 : 0;            // 32 K scales + 32 V scales
+  static constexpr int STAGE = 2 * KBYTES + SCBYTES;
+  static constexpr int IPS = 2 * NI + (FP8 ? 1 : 0);       // vector-memory instructions per stage
+};
+
+template <typename QT> struct Mma;
+template <> struct Mma<bf16_tag> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  }
+  static __device__ __forceinline__ uint32_t from_fp8(uint32_t w, bool hi) {
+    bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, r);
+  }
+};
+template <> struct Mma<fp16_tag> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    return (uint32_t)f32_to_fp16_bits(lo) | ((uint32_t)f32_to_fp16_bits(hi) << 16);
+  }
+  static __device__ __forceinline__ uint32_t from_fp8(uint32_t w, bool hi) {
+    f16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, r);
+  }
+};
+
+// 8 fp8 bytes (two dwords) -> 8 16-bit elements (four dwords), element order preserved.
+template <typename QT> __device__ __forceinline__ u32x4 widen8(uint32_t w0, uint32_t w1) {
+  u32x4 r;
+  r[0] = Mma<QT>::from_fp8(w0, false);
+  r[1] = Mma<QT>::from_fp8(w0, true);
+  r[2] = Mma<QT>::from_fp8(w1, false);
+  r[3] = Mma<QT>::from_fp8(w1, true);
+  return r;
+}
+
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const char* uni_ptr(const char* p) {
+  uint64_t v = (uint64_t)p;
+  uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const char*)(((uint64_t)hi << 32) | lo);
+}
+
+// Direct-to-LDS loads.  Issued through inline asm so that the waits are placed by hand (s_waitcnt vmcnt
+// below): a stage may be consumed while later stages are still in flight.  M0 carries the LDS destination
+// of lane 0; lane l lands at M0 + l*16 (or l*4).  One wait state is required between the M0 write and the load.
+__device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const char* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void dma4(uint32_t lds_addr, const void* vaddr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(vaddr) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+__device__ __forceinline__ float group_max(float x) {  // over the four 16-lane groups
+  x = fmaxf(x, __shfl_xor(x, 16, 64));
+  return fmaxf(x, __shfl_xor(x, 32, 64));
+}
+__device__ __forceinline__ float group_sum(float x) {
+  x += __shfl_xor(x, 16, 64);
+  return x + __shfl_xor(x, 32, 64);
+}
+
+__device__ __forceinline__ int units_of(int len) { return (len + kCT - 1) / kCT; }
+
+// Which partition holds global tile index u, for bounds u0(p) = floor(p*T/NP).
+__device__ __forceinline__ int part_of(int64_t u, int64_t T, int64_t NP) { return (int)(((u + 1) * NP - 1) / T); }
+__device__ __forceinline__ int part_begin(int64_t p, int64_t T, int64_t NP) { return (int)(p * T / NP); }
+
+// Position in the tile stream: sequence b, tile j of nt, plus the logical page / in-page offset of tile j.
+struct Cursor {
+  int b, j, nt, len, pg, off;
+};
+
+template <bool PS16>
+__device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int page_size) {
+  c.j++;
+  if (c.j < c.nt) {
+    if (PS16) {
+      c.pg += 2;
+    } else {
+      c.off += kCT;
+      if (c.off >= page_size) {
+        c.off = 0;
+        c.pg++;
+      }
+    }
+    return;
+  }
+  c.j = 0;
+  c.pg = 0;
+  c.off = 0;
+  do {
+    c.b++;
+    if (c.b >= batch) {
+      c.nt = 0;
+      c.len = 0;
+      return;
+    }
+    c.len = uni(seqlens[c.b]);
+    c.nt = units_of(c.len);
+  } while (c.nt == 0);
+}
+
+// ------------------------------------------------------------------------------------------------------
+template <typename QT, typename KVT, int NRB, int NS, bool SOFTCAP, bool PS16>
+__global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+  using G = Geom<KVT>;
+  constexpr bool FP8 = G::FP8;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const int wave = uni(threadIdx.x >> 6);
+  const int gw = blockIdx.x * kNW + wave;
+  const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
+  const int per_part = p.heads_kv * n_rg;
+  const int part = gw / per_part;
+  const int kvh = (gw - part * per_part) / n_rg;
+  const int rg = gw - part * per_part - kvh * n_rg;
+  const int64_t NP = p.n_parts;
+
+  // ---- tile-stream bookkeeping: total tiles, this partition's range, first sequence of the range ------
+  int T = 0;
+  for (int base = 0; base < p.batch; base += 64) {
+    int b = base + lane;
+    int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) n += __shfl_xor(n, m, 64);
+    T += n;
+  }
+  T = uni(T);
+  if (gw == 0) {  // exclusive prefix of tiles per sequence, for the combine kernel
+    int carry = 0;
+    for (int base = 0; base < p.batch; base += 64) {
+      int b = base + lane;
+      int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+      int incl = n;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        int t = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += t;
+      }
+      if (b < p.batch) ws_prefix[b] = carry + incl - n;
+      carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) ws_prefix[p.batch] = T;
+  }
+  if (part >= p.n_parts || T == 0) return;
+  const int u0 = part_begin(part, T, NP), u1 = part_begin(part + 1, T, NP);
+  const int n_units = u1 - u0;
+  if (n_units <= 0) return;
+
+  Cursor start;
+  {
+    int carry = 0, b0 = -1, pre0 = 0;
+    for (int base = 0; base < p.batch && b0 < 0; base += 64) {
+      int b = base + lane;
+      int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+      int incl = n;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        int t = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += t;
+      }
+      uint64_t hit = __ballot(carry + incl > u0);
+      if (hit) {
+        int idx = __ffsll((unsigned long long)hit) - 1;
+        b0 = base + idx;
+        pre0 = carry + __shfl(incl - n, idx, 64);
+      }
+      carry += __shfl(incl, 63, 64);
+    }
+    b0 = uni(b0);
+    pre0 = uni(pre0);
+    start.b = b0;
+    start.len = uni(p.seqlens[b0]);
+    start.nt = units_of(start.len);
+    start.j = u0 - pre0;
+    if (PS16) {
+      start.pg = 2 * start.j;
+      start.off = 0;
+    } else {
+      int tok = start.j * kCT;
+      start.pg = tok / p.page_size;
+      start.off = tok - start.pg * p.page_size;
+    }
+  }
+
+  // ---- loop-invariant lane constants ------------------------------------------------------------------
+  const int64_t row_stride = (int64_t)p.heads_kv * G::ROW;  // bytes between consecutive tokens of the pool
+  const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + wave * (NS * G::STAGE);
+
+  // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
+  // t = i*TPI + l/LPT (LPT lanes per token row), 16-byte slot l%LPT of that row.  The chunk fetched into
+  // slot s of token t is s ^ f(t), with f chosen per operand so that the MFMA-layout reads are conflict free:
+  //   bf16 K: f = t%16          bf16 V: f = 2*(t%8)
+  //   fp8  K: f = (t/2)%8       fp8  V: f = (t/2)%4 + 4*((t/16)%2)
+  constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
+  const int ts = lane / LPT, slot = lane % LPT;
+  uint32_t voff_k[FP8 ? 2 : 4], voff_v[2];
+  if (!FP8) {
+#pragma unroll
+    for (int v = 0; v < 4; v++) voff_k[v] = (uint32_t)(ts * row_stride) + ((slot ^ ((4 * v + ts) & 15)) << 4);
+#pragma unroll
+    for (int v = 0; v < 2; v++) voff_v[v] = (uint32_t)(ts * row_stride) + ((slot ^ (2 * ((4 * v + ts) & 7))) << 4);
+  } else {
+#pragma unroll
+    for (int v = 0; v < 2; v++) voff_k[v] = (uint32_t)(ts * row_stride) + ((slot ^ ((4 * v + ts / 2) & 7)) << 4);
+#pragma unroll
+    for (int v = 0; v < 2; v++) voff_v[v] = (uint32_t)(ts * row_stride) + ((slot ^ (((ts / 2) & 3) + 4 * v)) << 4);
+  }
+  auto k_variant = [](int i) { return FP8 ? (i & 1) : (i & 3); };
+  auto v_variant = [](int i) { return FP8 ? ((i >> 1) & 1) : (i & 1); };
+
+  // LDS read addresses (relative to a stage's K, V region), see the header comment for the layouts.
+  uint32_t ka[FP8 ? 2 : 4], va[8];
+  if (!FP8) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) ka[j] = (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
+    const int jj = c, tk = 4 * g + jj / 4;  // transpose read: lane supplies row tk, 8 bytes at column group jj%4
+#pragma unroll
+    for (int db = 0; db < 8; db++) va[db] = (uint32_t)((tk * 256 + (tk & 7) * 32 + (jj & 3) * 8) ^ (db * 32));
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2; j++) ka[j] = (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
+    const int jj = c, r8 = jj >> 1;  // transpose read of bytes: lane supplies row r8 of 8, 8 bytes at half jj%2
+    const int tk = r8 < 4 ? 4 * g + r8 : 16 + 4 * g + (r8 - 4);
+    const int fv = ((tk >> 1) & 3) + 4 * ((tk >> 4) & 1);
+#pragma unroll
+    for (int db = 0; db < 8; db++) va[db] = (uint32_t)((tk * 128 + fv * 16 + (jj & 1) * 8) ^ (db * 16));
+  }
+
+  // ---- stage issue --------------------------------------------------------------------------------------
+  const char* const kpool = (const char*)p.k;
+  const char* const vpool = (const char*)p.v;
+  auto phys_page = [&](const Cursor& cu, int pg) -> int64_t {
+    int64_t e = uni(p.block_table[(int64_t)cu.b * p.bt_row_stride + pg]);
+    return e < 0 ? 0 : (e >= p.n_pages ? p.n_pages - 1 : e);
+  };
+  auto issue = [&](const Cursor& cu, int slot_idx) {
+    const int tok0 = cu.j * kCT;
+    const int nvalid = min(kCT, cu.len - tok0);  // >= 1
+    int64_t ptok0, ptok1 = 0;                    // physical token of the stage's first token (and of its 2nd page)
+    if (PS16) {
+      int last_pg = (cu.len - 1) >> 4;
+      ptok0 = phys_page(cu, cu.pg) * 16;
+      ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
+    } else {
+      ptok0 = phys_page(cu, cu.pg) * p.page_size + cu.off;
+    }
+    const uint32_t lds = lds_wave + slot_idx * G::STAGE;
+    const int64_t head_off = (int64_t)kvh * G::ROW;
+    const bool full = nvalid == kCT;
+    const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
+#pragma unroll
+    for (int i = 0; i < G::NI; i++) {
+      int si = full ? i : min(i, i_last);  // source instruction (tail stages re-read the last valid rows)
+      int64_t ptok;
+      if (PS16) {
+        constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
+        ptok = (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI;
+      } else {
+        ptok = ptok0 + si * G::TPI;
+      }
+      int64_t goff = ptok * row_stride + head_off;
+      uint32_t vk = voff_k[k_variant(i)], vv = voff_v[v_variant(i)];
+      if (!full && si == i_last && ts > t_last) {
+        uint32_t back = (uint32_t)((ts - t_last) * row_stride);
+        vk -= back;
+        vv -= back;
+      }
+      dma16_nt(lds + i * 1024, vk, kpool + goff);
+      dma16_nt(lds + G::KBYTES + i * 1024, vv, vpool + goff);
+    }
+    if (FP8) {
+      int tk = min(lane & 31, nvalid - 1);
+      int64_t ptok = PS16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
+      const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + ptok * p.heads_kv + kvh;
+      dma4(lds + 2 * G::KBYTES, sp);
+    }
+  };
+
+  // ---- per-segment state ----------------------------------------------------------------------------------
+  u32x4 qreg[NRB][4];
+  f32x4 o_acc[NRB][8];
+  float m_run[NRB], l_run[NRB];
+  int limit[NRB];
+  const int qoff = (p.causal && p.q_len > 1) ? p.q_len - 1 : 0;
+
+  auto begin_segment = [&](const Cursor& cu) {
+#pragma unroll
+    for (int rb = 0; rb < NRB; rb++) {
+      int r = rg * (16 * NRB) + rb * 16 + c;
+      bool valid = r < p.rows;
+      int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
+      const char* qp = (const char*)p.q + ((((int64_t)cu.b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) * 2;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        // head elements this lane contributes to k-step j: 8 consecutive ones, matching the K operand
+        int d0 = FP8 ? 64 * (j >> 1) + 16 * g + 8 * (j & 1) : 32 * j + 8 * g;
+        u32x4 z = {0, 0, 0, 0};
+        qreg[rb][j] = valid ? *(const u32x4*)(qp + d0 * 2) : z;
+      }
+      limit[rb] = valid ? ((p.causal && p.q_len > 1) ? cu.len - p.q_len + s + 1 : cu.len) : 0;
+      m_run[rb] = kNegFloor;
+      l_run[rb] = 0.f;
+#pragma unroll
+      for (int db = 0; db < 8; db++) o_acc[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+
+  auto compute = [&](const Cursor& cu, int slot_idx) {
+    const uint32_t kl = lds_wave + slot_idx * G::STAGE;
+    const uint32_t vl = kl + G::KBYTES;
+    const int tok0 = cu.j * kCT;
+    f32x4 s_acc[2][NRB];
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+      for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // S^T = K . Q^T
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) {
+      if (!FP8) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          u32x4 a = *LDS_AT(u32x4, kl + tb * 4096 + ka[j]);
+#pragma unroll
+          for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = Mma<QT>::run(a, qreg[rb][j], s_acc[tb][rb]);
+        }
+      } else {
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+          u32x4 raw = *LDS_AT(u32x4, kl + tb * 2048 + ka[jj]);
+          u32x4 a0 = widen8<QT>(raw[0], raw[1]), a1 = widen8<QT>(raw[2], raw[3]);
+#pragma unroll
+          for (int rb = 0; rb < NRB; rb++) {
+            s_acc[tb][rb] = Mma<QT>::run(a0, qreg[rb][2 * jj], s_acc[tb][rb]);
+            s_acc[tb][rb] = Mma<QT>::run(a1, qreg[rb][2 * jj + 1], s_acc[tb][rb]);
+          }
+        }
+      }
+    }
+    f32x4 ksc[2], vsc[2];
+    if (FP8) {
+      const uint32_t sl = kl + 2 * G::KBYTES;
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++) {
+        ksc[tb] = *LDS_AT(f32x4, sl + (16 * tb + 4 * g) * 4);
+        vsc[tb] = *LDS_AT(f32x4, sl + 128 + (16 * tb + 4 * g) * 4);
+      }
+    }
+    const bool need_mask = tok0 + kCT > cu.len - qoff;
+    u32x4 pk[NRB];
+    float alpha[NRB];
+    bool any_rescale = false;
+#pragma unroll
+    for (int rb = 0; rb < NRB; rb++) {
+      float x[2][4];
+      float mt = -INFINITY;
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float s = s_acc[tb][rb][i];
+          if (FP8) s *= ksc[tb][i];
+          float v = to_logit2<SOFTCAP>(s, p.score_scale, p.cap_log2e, p.inv_cap_scale);
+          if (need_mask && tok0 + 16 * tb + 4 * g + i >= limit[rb]) v = -INFINITY;
+          x[tb][i] = v;
+          mt = fmaxf(mt, v);
+        }
+      mt = group_max(mt);
+      float m_new = fmaxf(m_run[rb], mt);
+      alpha[rb] = exp2f(m_run[rb] - m_new);
+      m_run[rb] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float pr = exp2f(x[tb][i] - m_new);
+          psum += pr;
+          x[tb][i] = FP8 ? pr * vsc[tb][i] : pr;
+        }
+      l_run[rb] = l_run[rb] * alpha[rb] + psum;
+      pk[rb][0] = Mma<QT>::pack(x[0][0], x[0][1]);
+      pk[rb][1] = Mma<QT>::pack(x[0][2], x[0][3]);
+      pk[rb][2] = Mma<QT>::pack(x[1][0], x[1][1]);
+      pk[rb][3] = Mma<QT>::pack(x[1][2], x[1][3]);
+      any_rescale |= alpha[rb] != 1.0f;
+    }
+    if (__any(any_rescale)) {
+#pragma unroll
+      for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+        for (int db = 0; db < 8; db++) o_acc[rb][db] *= alpha[rb];
+    }
+    // O^T += V^T . P^T
+#pragma unroll
+    for (int db = 0; db < 8; db++) {
+      u32x4 a;
+      if (!FP8) {
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vl + va[db]));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vl + 4096 + va[db]));
+        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        a = u32x4{l2[0], l2[1], h2[0], h2[1]};
+      } else {
+        i32x2 r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vl + va[db]));
+        a = widen8<QT>((uint32_t)r[0], (uint32_t)r[1]);
+      }
+#pragma unroll
+      for (int rb = 0; rb < NRB; rb++) o_acc[rb][db] = Mma<QT>::run(a, pk[rb], o_acc[rb][db]);
+    }
+  };
+
+  auto end_segment = [&](const Cursor& cu, bool complete, int which) {
+#pragma unroll
+    for (int rb = 0; rb < NRB; rb++) {
+      int r = rg * (16 * NRB) + rb * 16 + c;
+      float l_tot = group_sum(l_run[rb]);
+      float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+      if (r >= p.rows) continue;
+      if (complete) {
+        int s = r / p.group, gi = r - s * p.group;
+        uint16_t* op = (uint16_t*)p.out + (((int64_t)cu.b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD;
+#pragma unroll
+        for (int db = 0; db < 8; db++) {
+          f32x4 o = o_acc[rb][db] * inv;
+          u32x2 w;
+          w[0] = Mma<QT>::pack(o[0], o[1]);
+          w[1] = Mma<QT>::pack(o[2], o[3]);
+          *(u32x2*)(op + 16 * db + 4 * g) = w;
+        }
+      } else {
+        int64_t grow = ((int64_t)(2 * part + which) * p.heads_kv + kvh) * p.rows + r;
+        float* pp = p.part_o + grow * kD;
+#pragma unroll
+        for (int db = 0; db < 8; db++) *(f32x4*)(pp + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+        if (g == 0) p.part_lse[grow] = l_tot > 0.f ? m_run[rb] + log2f(l_tot) : -INFINITY;
+      }
+    }
+  };
+
+  // ---- software pipeline over this wave's tiles ---------------------------------------------------------
+  Cursor ci = start, cc = start;
+  int issued = 0;
+  for (; issued < NS - 1 && issued < n_units; ++issued) {
+    issue(ci, issued % NS);
+    cursor_next<PS16>(ci, p.seqlens, p.batch, p.page_size);
+  }
+  bool seg_open = false;
+  int seg_first_j = 0, seg_count = 0;
+  for (int u = 0; u < n_units; ++u) {
+    if (issued < n_units) {
+      issue(ci, issued % NS);
+      cursor_next<PS16>(ci, p.seqlens, p.batch, p.page_size);
+      ++issued;
+    }
+    if (!seg_open) {
+      begin_segment(cc);
+      seg_open = true;
+      seg_first_j = cc.j;
+    }
+    const int ahead = issued - u - 1;  // stages issued after the one consumed now
+    if (ahead >= 3) wait_vmcnt<(NS > 3 ? 3 : NS - 1) * G::IPS>();
+    else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * G::IPS>();
+    else if (ahead == 1) wait_vmcnt<G::IPS>();
+    else wait_vmcnt<0>();
+    compute(cc, u % NS);
+    const bool last_of_seq = cc.j == cc.nt - 1;
+    if (last_of_seq || u == n_units - 1) {
+      end_segment(cc, seg_first_j == 0 && last_of_seq, seg_count == 0 ? 0 : 1);
+      seg_open = false;
+      ++seg_count;
+    }
+    cursor_next<PS16>(cc, p.seqlens, p.batch, p.page_size);
+  }
+}
+
+// Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
+// grid (heads_kv*rows, batch), 128 threads (one per head element).
+template <typename QT>
+__global__ __launch_bounds__(kD) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix) {
+  const int b = blockIdx.y, row_all = blockIdx.x, d = threadIdx.x;
+  const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
+  const int s = r / p.group, gi = r - s * p.group;
+  uint16_t* op = (uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD + d;
+  const int len = p.seqlens[b];
+  const int nt = units_of(len);
+  if (nt == 0) {
+    *op = 0;
+    return;
+  }
+  const int64_t T = ws_prefix[p.batch], NP = p.n_parts, pre = ws_prefix[b];
+  const int p_first = part_of(pre, T, NP), p_last = part_of(pre + nt - 1, T, NP);
+  if (p_first == p_last) return;  // one wave covered the whole sequence and wrote the output itself
+  const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
+  auto slot_of = [&](int pp) -> int64_t {
+    int which = (pp == p_first && part_begin(pp, T, NP) != pre) ? 1 : 0;
+    return (int64_t)(2 * pp + which) * rows_all + row_all;
+  };
+  // with fewer tiles than partitions some partitions in between own no tile and wrote nothing
+  auto owns_tiles = [&](int pp) { return part_begin(pp + 1, T, NP) > part_begin(pp, T, NP); };
+  float M = -INFINITY;
+  for (int pp = p_first; pp <= p_last; pp++)
+    if (owns_tiles(pp)) M = fmaxf(M, p.part_lse[slot_of(pp)]);
+  float W = 0.f, A = 0.f;
+  if (M > -INFINITY) {
+    for (int pp = p_first; pp <= p_last; pp++) {
+      if (!owns_tiles(pp)) continue;
+      int64_t sl = slot_of(pp);
+      float w = exp2f(p.part_lse[sl] - M);
+      W += w;
+      A += w * p.part_o[sl * kD + d];
+    }
+  }
+  *op = f32_to_elem_bits<QT>(W > 0.f ? A / W : 0.f);
+}
+
+template <typename KVT> constexpr int stages_for() { return Geom<KVT>::FP8 ? 3 : 2; }
+
+template <typename QT, typename KVT, int NRB>
+const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
+  constexpr int NS = stages_for<KVT>();
+  const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
+  const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
+  const int grid = (int)((waves + kNW - 1) / kNW);
+  const size_t lds = (size_t)kNW * NS * Geom<KVT>::STAGE;
+  const bool ps16 = p.page_size == 16, cap = p.softcap > 0.f;
+#define MI355_LAUNCH(SC, P16)                                                                                         \
+  do {                                                                                                                \
+    auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, SC, P16>;                                                  \
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
+    if (e != hipSuccess) return hipGetErrorString(e);                                                                 \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);                                       \
+  } while (0)
+  if (cap && ps16) MI355_LAUNCH(true, true);
+  else if (cap) MI355_LAUNCH(true, false);
+  else if (ps16) MI355_LAUNCH(false, true);
+  else MI355_LAUNCH(false, false);
+#undef MI355_LAUNCH
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hipGetErrorString(e);
+  hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(kD), 0, s, p, ws_prefix);
+  e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
+int row_blocks_for(int rows) { return rows <= 16 ? 1 : (rows <= 32 ? 2 : 4); }
+
+template <typename QT, typename KVT>
+const char* launch_t2(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
+  switch (row_blocks_for(p.rows)) {
+    case 1: return launch_t3<QT, KVT, 1>(p, ws_prefix, s);
+    case 2: return launch_t3<QT, KVT, 2>(p, ws_prefix, s);
+    default: return launch_t3<QT, KVT, 4>(p, ws_prefix, s);
+  }
+}
+
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+}  // namespace
+
+bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap) {
+  (void)q_len; (void)heads; (void)heads_kv; (void)softcap;
+  if (dim != kD) return false;
+  if (!(page_size == 16 || page_size % kCT == 0)) return false;
+  if (kv_dtype != MI355_DT_FP8_E4M3FN && kv_dtype != q_dtype) return false;
+  return true;
+}
+
+// Number of equal ranges the tile stream is cut into: one wave per (range, kv head, row group), sized so
+// that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
+int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
+  const int nrb = row_blocks_for(rows);
+  const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
+  const int wgs_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 1 : 1;
+  const int64_t waves = (int64_t)kNumCU * wgs_per_cu * kNW;
+  int64_t parts = waves / ((int64_t)heads_kv * n_rg);
+  return parts < 1 ? 1 : (int)parts;
+}
+
+// [part_o: 2*n_parts slots x heads_kv*rows x dim fp32][part_lse: 2*n_parts x heads_kv*rows fp32][prefix: batch+1 int32]
+size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int batch) {
+  size_t slots = (size_t)2 * n_parts * heads_kv * rows;
+  return align256(slots * dim * sizeof(float)) + align256(slots * sizeof(float)) + align256((size_t)(batch + 1) * sizeof(int));
+}
+
+const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, hipStream_t s) {
+  DecodeParams p = p_in;
+  size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
+  char* ws = (char*)p_in.part_o;
+  p.part_o = (float*)ws;
+  p.part_lse = (float*)(ws + align256(slots * kD * sizeof(float)));
+  int* ws_prefix = (int*)(ws + align256(slots * kD * sizeof(float)) + align256(slots * sizeof(float)));
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag>(p, ws_prefix, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag>(p, ws_prefix, s);
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag>(p, ws_prefix, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag>(p, ws_prefix, s);
+  return "MFMA kernel: unsupported (q_dtype, kv_dtype) pair";
+}
+
 }  // namespace mi355
