@@ -102,23 +102,41 @@ __device__ __forceinline__ const char* uni_ptr(const char* p) {
 
 // Direct-to-LDS loads.  Issued through inline asm so that the waits are placed by hand (s_waitcnt vmcnt
 // below): a stage may be consumed while later stages are still in flight.  M0 carries the LDS destination
-// of lane 0; lane l lands at M0 + l*16 (or l*4).  One wait state is required between the M0 write and the load.
+// of lane 0; lane l lands at M0 + l*16 (or l*4).  The scalar operands are pinned to SGPRs here because a
+// wave-uniform value may still have been computed on the vector ALU; the s_nop covers both the M0 write ->
+// LDS-DMA wait state and the five wait states a VMEM instruction needs after a VALU write of its SGPR base,
+// which the compiler's hazard recogniser cannot insert inside an asm block.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const char* sbase) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  sbase = uni_ptr(sbase);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 __device__ __forceinline__ void dma4(uint32_t lds_addr, const void* vaddr) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(vaddr) : "memory");
 }
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-__device__ __forceinline__ float group_max(float x) {  // over the four 16-lane groups
-  x = fmaxf(x, __shfl_xor(x, 16, 64));
-  return fmaxf(x, __shfl_xor(x, 32, 64));
+// Reductions over the four 16-lane groups of a wave (lanes c, c+16, c+32, c+48) with the gfx950 lane-swap
+// instructions: v_permlane16_swap exchanges odd 16-lane rows of its first operand with even rows of the
+// second, v_permlane32_swap exchanges the upper half of the first with the lower half of the second.  Fed the
+// same value twice they return (x of the even partner, x of the odd partner), so one max/add finishes a step
+// without touching the LDS crossbar.
+__device__ __forceinline__ float group_max(float x) {
+  u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float group_sum(float x) {
-  x += __shfl_xor(x, 16, 64);
-  return x + __shfl_xor(x, 32, 64);
+  u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// v_exp_f32: exp2 without the denormal-range fix-up of exp2f (arguments here are <= 0 or -inf; a result
+// below 2^-126 may flush to zero, which is what a softmax weight that small should be).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ int units_of(int len) { return (len + kCT - 1) / kCT; }
 
@@ -131,11 +149,10 @@ struct Cursor {
   int b, j, nt, len, pg, off;
 };
 
-template <bool PS16>
-__device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int page_size) {
+__device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int page_size, bool ps16) {
   c.j++;
   if (c.j < c.nt) {
-    if (PS16) {
+    if (ps16) {
       c.pg += 2;
     } else {
       c.off += kCT;
@@ -162,7 +179,9 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------------
-template <typename QT, typename KVT, int NRB, int NS, bool SOFTCAP, bool PS16>
+template <int V> struct IntC { static constexpr int value = V; };
+
+template <typename QT, typename KVT, int NRB, int NS>
 __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
@@ -174,10 +193,13 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
   const int gw = blockIdx.x * kNW + wave;
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int per_part = p.heads_kv * n_rg;
-  const int part = gw / per_part;
-  const int kvh = (gw - part * per_part) / n_rg;
-  const int rg = gw - part * per_part - kvh * n_rg;
+  // integer division runs on the vector ALU; pin the results to scalar registers so that everything derived
+  // from them (pool base pointers, LDS bases) is scalar arithmetic
+  const int part = uni(gw / per_part);
+  const int kvh = uni((gw - part * per_part) / n_rg);
+  const int rg = uni(gw - part * per_part - kvh * n_rg);
   const int64_t NP = p.n_parts;
+  const bool ps16 = p.page_size == 16;
 
   // ---- tile-stream bookkeeping: total tiles, this partition's range, first sequence of the range ------
   int T = 0;
@@ -236,18 +258,18 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
     start.len = uni(p.seqlens[b0]);
     start.nt = units_of(start.len);
     start.j = u0 - pre0;
-    if (PS16) {
+    if (ps16) {
       start.pg = 2 * start.j;
       start.off = 0;
     } else {
       int tok = start.j * kCT;
-      start.pg = tok / p.page_size;
+      start.pg = uni(tok / p.page_size);
       start.off = tok - start.pg * p.page_size;
     }
   }
 
   // ---- loop-invariant lane constants ------------------------------------------------------------------
-  const int64_t row_stride = (int64_t)p.heads_kv * G::ROW;  // bytes between consecutive tokens of the pool
+  const uint32_t row_stride = (uint32_t)p.heads_kv * G::ROW;  // bytes between consecutive tokens of the pool
   const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + wave * (NS * G::STAGE);
 
   // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
@@ -256,85 +278,103 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
   //   bf16 K: f = t%16          bf16 V: f = 2*(t%8)
   //   fp8  K: f = (t/2)%8       fp8  V: f = (t/2)%4 + 4*((t/16)%2)
   constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
+  constexpr int NKV = FP8 ? 2 : 4;  // distinct per-lane offset patterns of the K instructions
   const int ts = lane / LPT, slot = lane % LPT;
-  uint32_t voff_k[FP8 ? 2 : 4], voff_v[2];
+  uint32_t voff_k[NKV], voff_v[2];
   if (!FP8) {
 #pragma unroll
-    for (int v = 0; v < 4; v++) voff_k[v] = (uint32_t)(ts * row_stride) + ((slot ^ ((4 * v + ts) & 15)) << 4);
+    for (int v = 0; v < 4; v++) voff_k[v] = ts * row_stride + ((slot ^ ((4 * v + ts) & 15)) << 4);
 #pragma unroll
-    for (int v = 0; v < 2; v++) voff_v[v] = (uint32_t)(ts * row_stride) + ((slot ^ (2 * ((4 * v + ts) & 7))) << 4);
+    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (2 * ((4 * v + ts) & 7))) << 4);
   } else {
 #pragma unroll
-    for (int v = 0; v < 2; v++) voff_k[v] = (uint32_t)(ts * row_stride) + ((slot ^ ((4 * v + ts / 2) & 7)) << 4);
+    for (int v = 0; v < 2; v++) voff_k[v] = ts * row_stride + ((slot ^ ((4 * v + ts / 2) & 7)) << 4);
 #pragma unroll
-    for (int v = 0; v < 2; v++) voff_v[v] = (uint32_t)(ts * row_stride) + ((slot ^ (((ts / 2) & 3) + 4 * v)) << 4);
+    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (((ts / 2) & 3) + 4 * v)) << 4);
   }
-  auto k_variant = [](int i) { return FP8 ? (i & 1) : (i & 3); };
-  auto v_variant = [](int i) { return FP8 ? ((i >> 1) & 1) : (i & 1); };
 
-  // LDS read addresses (relative to a stage's K, V region), see the header comment for the layouts.
-  uint32_t ka[FP8 ? 2 : 4], va[8];
+  // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
+  constexpr int NKA = FP8 ? 2 : 4;
+  uint32_t kaddr[NKA], vaddr[8];
   if (!FP8) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) ka[j] = (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
-    const int jj = c, tk = 4 * g + jj / 4;  // transpose read: lane supplies row tk, 8 bytes at column group jj%4
+    for (int j = 0; j < 4; j++) kaddr[j] = lds_wave + (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
+    const int tk = 4 * g + c / 4;  // transpose read: lane supplies row tk, 8 bytes at column group c%4
 #pragma unroll
-    for (int db = 0; db < 8; db++) va[db] = (uint32_t)((tk * 256 + (tk & 7) * 32 + (jj & 3) * 8) ^ (db * 32));
+    for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 256 + (tk & 7) * 32 + (c & 3) * 8) ^ (db * 32));
   } else {
 #pragma unroll
-    for (int j = 0; j < 2; j++) ka[j] = (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
-    const int jj = c, r8 = jj >> 1;  // transpose read of bytes: lane supplies row r8 of 8, 8 bytes at half jj%2
+    for (int j = 0; j < 2; j++) kaddr[j] = lds_wave + (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
+    const int r8 = c >> 1;  // transpose read of bytes: lane supplies row r8 of 8, 8 bytes at half c%2
     const int tk = r8 < 4 ? 4 * g + r8 : 16 + 4 * g + (r8 - 4);
     const int fv = ((tk >> 1) & 3) + 4 * ((tk >> 4) & 1);
 #pragma unroll
-    for (int db = 0; db < 8; db++) va[db] = (uint32_t)((tk * 128 + fv * 16 + (jj & 1) * 8) ^ (db * 16));
+    for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 128 + fv * 16 + (c & 1) * 8) ^ (db * 16));
   }
+  const uint32_t saddr = lds_wave + 2 * G::KBYTES + (uint32_t)(4 * g) * 4;  // scales of tokens 4g.. (fp8)
 
   // ---- stage issue --------------------------------------------------------------------------------------
-  const char* const kpool = (const char*)p.k;
-  const char* const vpool = (const char*)p.v;
-  auto phys_page = [&](const Cursor& cu, int pg) -> int64_t {
-    int64_t e = uni(p.block_table[(int64_t)cu.b * p.bt_row_stride + pg]);
+  const char* const kpool = uni_ptr((const char*)p.k + (int64_t)kvh * G::ROW);
+  const char* const vpool = uni_ptr((const char*)p.v + (int64_t)kvh * G::ROW);
+  // Block-table entries of the sequence being issued live in one VGPR: lane l holds logical page
+  // bt_base + l.  A stage fetches its entry with v_readlane, so the steady-state loop contains no
+  // compiler-visible memory load (whose vmcnt wait would drain the direct-to-LDS pipeline); the register
+  // is refilled once per 64 pages.
+  int bt_reg = 0, bt_base = 0, bt_seq = -1;
+  auto phys_page = [&](const Cursor& cu, int pg) __attribute__((always_inline)) -> int64_t {
+    if (cu.b != bt_seq || pg < bt_base || pg >= bt_base + 64) {
+      bt_seq = cu.b;
+      bt_base = pg;
+      int last_pg = uni((cu.len - 1) / p.page_size);  // never read past the entries the sequence owns
+      bt_reg = p.block_table[(int64_t)cu.b * p.bt_row_stride + min(pg + lane, last_pg)];
+    }
+    int64_t e = __builtin_amdgcn_readlane(bt_reg, pg - bt_base);
     return e < 0 ? 0 : (e >= p.n_pages ? p.n_pages - 1 : e);
   };
-  auto issue = [&](const Cursor& cu, int slot_idx) {
+  auto issue = [&](const Cursor& cu, int slot_idx) __attribute__((always_inline)) {
     const int tok0 = cu.j * kCT;
     const int nvalid = min(kCT, cu.len - tok0);  // >= 1
-    int64_t ptok0, ptok1 = 0;                    // physical token of the stage's first token (and of its 2nd page)
-    if (PS16) {
+    const uint32_t lds = lds_wave + slot_idx * G::STAGE;
+    int64_t ptok0, ptok1 = 0;  // physical token of the stage's first token (and of its second 16-token page)
+    if (ps16) {
       int last_pg = (cu.len - 1) >> 4;
       ptok0 = phys_page(cu, cu.pg) * 16;
       ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
     } else {
       ptok0 = phys_page(cu, cu.pg) * p.page_size + cu.off;
     }
-    const uint32_t lds = lds_wave + slot_idx * G::STAGE;
-    const int64_t head_off = (int64_t)kvh * G::ROW;
-    const bool full = nvalid == kCT;
-    const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
+    if (nvalid == kCT && !ps16) {
+      // common case: 32 valid tokens inside one page -- straight-line, two scalar adds per instruction
+      const char* kb = kpool + ptok0 * row_stride;
+      const char* vb = vpool + ptok0 * row_stride;
+      const uint32_t step = G::TPI * row_stride;
 #pragma unroll
-    for (int i = 0; i < G::NI; i++) {
-      int si = full ? i : min(i, i_last);  // source instruction (tail stages re-read the last valid rows)
-      int64_t ptok;
-      if (PS16) {
-        constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
-        ptok = (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI;
-      } else {
-        ptok = ptok0 + si * G::TPI;
+      for (int i = 0; i < G::NI; i++) {
+        dma16_nt(lds + i * 1024, voff_k[FP8 ? (i & 1) : (i & 3)], kb + i * step);
+        dma16_nt(lds + G::KBYTES + i * 1024, voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)], vb + i * step);
       }
-      int64_t goff = ptok * row_stride + head_off;
-      uint32_t vk = voff_k[k_variant(i)], vv = voff_v[v_variant(i)];
-      if (!full && si == i_last && ts > t_last) {
-        uint32_t back = (uint32_t)((ts - t_last) * row_stride);
-        vk -= back;
-        vv -= back;
+    } else {
+      // tail of a sequence and/or 16-token pages: rows past the valid ones re-read the last valid row, so
+      // nothing outside (block_table, real_seqlen_kv) is ever touched
+      const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
+      constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
+#pragma unroll
+      for (int i = 0; i < G::NI; i++) {
+        int si = min(i, i_last);
+        int64_t ptok = ps16 ? (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI : ptok0 + si * G::TPI;
+        uint32_t vk = voff_k[FP8 ? (i & 1) : (i & 3)], vv = voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)];
+        if (si == i_last && ts > t_last) {
+          uint32_t back = (uint32_t)(ts - t_last) * row_stride;
+          vk -= back;
+          vv -= back;
+        }
+        dma16_nt(lds + i * 1024, vk, kpool + ptok * row_stride);
+        dma16_nt(lds + G::KBYTES + i * 1024, vv, vpool + ptok * row_stride);
       }
-      dma16_nt(lds + i * 1024, vk, kpool + goff);
-      dma16_nt(lds + G::KBYTES + i * 1024, vv, vpool + goff);
     }
     if (FP8) {
       int tk = min(lane & 31, nvalid - 1);
-      int64_t ptok = PS16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
+      int64_t ptok = ps16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
       const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + ptok * p.heads_kv + kvh;
       dma4(lds + 2 * G::KBYTES, sp);
     }
@@ -346,8 +386,9 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
   float m_run[NRB], l_run[NRB];
   int limit[NRB];
   const int qoff = (p.causal && p.q_len > 1) ? p.q_len - 1 : 0;
+  const bool softcap = p.softcap > 0.f;
 
-  auto begin_segment = [&](const Cursor& cu) {
+  auto begin_segment = [&](const Cursor& cu) __attribute__((always_inline)) {
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       int r = rg * (16 * NRB) + rb * 16 + c;
@@ -367,49 +408,72 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 #pragma unroll
       for (int db = 0; db < 8; db++) o_acc[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    // Make the query loads land here: an empty asm that "modifies" each register forces the compiler to put
+    // its own vmcnt wait in this (rare) block instead of in the steady-state loop, where such a wait would
+    // also wait for every direct-to-LDS load in flight.
+#pragma unroll
+    for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) asm volatile("" : "+v"(qreg[rb][j]));
   };
 
-  auto compute = [&](const Cursor& cu, int slot_idx) {
-    const uint32_t kl = lds_wave + slot_idx * G::STAGE;
-    const uint32_t vl = kl + G::KBYTES;
+  auto compute = [&](auto slot_c, const Cursor& cu) __attribute__((always_inline)) {
+    constexpr int SOFF = decltype(slot_c)::value * G::STAGE;
     const int tok0 = cu.j * kCT;
+    // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
+    u32x4 ka_op[2][4], va_op[8];
+    f32x4 ksc[2], vsc[2];
+    if (!FP8) {
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j] + (SOFF + tb * 4096));
+#pragma unroll
+      for (int db = 0; db < 8; db++) {
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + SOFF));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + (SOFF + 4096)));
+        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+      }
+    } else {
+      u32x4 kraw[2][2];
+      i32x2 vraw[8];
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) kraw[tb][jj] = *LDS_AT(u32x4, kaddr[jj] + (SOFF + tb * 2048));
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++) {
+        ksc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 64 * tb));
+        vsc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 128 + 64 * tb));
+      }
+#pragma unroll
+      for (int db = 0; db < 8; db++) vraw[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+          ka_op[tb][2 * jj] = widen8<QT>(kraw[tb][jj][0], kraw[tb][jj][1]);
+          ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
+        }
+#pragma unroll
+      for (int db = 0; db < 8; db++) va_op[db] = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
+    }
+    if (!FP8) __builtin_amdgcn_sched_barrier(0);
+    // ---- S^T = K . Q^T : the two 16-token blocks interleaved so dependent MFMAs are one apart -------------
     f32x4 s_acc[2][NRB];
 #pragma unroll
     for (int tb = 0; tb < 2; tb++)
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // S^T = K . Q^T
 #pragma unroll
-    for (int tb = 0; tb < 2; tb++) {
-      if (!FP8) {
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          u32x4 a = *LDS_AT(u32x4, kl + tb * 4096 + ka[j]);
+      for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-          for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = Mma<QT>::run(a, qreg[rb][j], s_acc[tb][rb]);
-        }
-      } else {
-#pragma unroll
-        for (int jj = 0; jj < 2; jj++) {
-          u32x4 raw = *LDS_AT(u32x4, kl + tb * 2048 + ka[jj]);
-          u32x4 a0 = widen8<QT>(raw[0], raw[1]), a1 = widen8<QT>(raw[2], raw[3]);
-#pragma unroll
-          for (int rb = 0; rb < NRB; rb++) {
-            s_acc[tb][rb] = Mma<QT>::run(a0, qreg[rb][2 * jj], s_acc[tb][rb]);
-            s_acc[tb][rb] = Mma<QT>::run(a1, qreg[rb][2 * jj + 1], s_acc[tb][rb]);
-          }
-        }
-      }
-    }
-    f32x4 ksc[2], vsc[2];
-    if (FP8) {
-      const uint32_t sl = kl + 2 * G::KBYTES;
-#pragma unroll
-      for (int tb = 0; tb < 2; tb++) {
-        ksc[tb] = *LDS_AT(f32x4, sl + (16 * tb + 4 * g) * 4);
-        vsc[tb] = *LDS_AT(f32x4, sl + 128 + (16 * tb + 4 * g) * 4);
-      }
-    }
+        for (int tb = 0; tb < 2; tb++) s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
+    // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
     const bool need_mask = tok0 + kCT > cu.len - qoff;
     u32x4 pk[NRB];
     float alpha[NRB];
@@ -417,28 +481,43 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       float x[2][4];
-      float mt = -INFINITY;
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           float s = s_acc[tb][rb][i];
           if (FP8) s *= ksc[tb][i];
-          float v = to_logit2<SOFTCAP>(s, p.score_scale, p.cap_log2e, p.inv_cap_scale);
-          if (need_mask && tok0 + 16 * tb + 4 * g + i >= limit[rb]) v = -INFINITY;
-          x[tb][i] = v;
-          mt = fmaxf(mt, v);
+          x[tb][i] = s;
         }
+      if (softcap) {
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[tb][i] = to_logit2<true>(x[tb][i], p.score_scale, p.cap_log2e, p.inv_cap_scale);
+      } else {
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[tb][i] *= p.score_scale;
+      }
+      if (need_mask) {  // only the last tile(s) of a sequence
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+            if (tok0 + 16 * tb + 4 * g + i >= limit[rb]) x[tb][i] = -INFINITY;
+      }
+      float mt = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])), fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
       mt = group_max(mt);
       float m_new = fmaxf(m_run[rb], mt);
-      alpha[rb] = exp2f(m_run[rb] - m_new);
+      alpha[rb] = fast_exp2(m_run[rb] - m_new);
       m_run[rb] = m_new;
       float psum = 0.f;
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          float pr = exp2f(x[tb][i] - m_new);
+          float pr = fast_exp2(x[tb][i] - m_new);
           psum += pr;
           x[tb][i] = FP8 ? pr * vsc[tb][i] : pr;
         }
@@ -455,25 +534,14 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 #pragma unroll
         for (int db = 0; db < 8; db++) o_acc[rb][db] *= alpha[rb];
     }
-    // O^T += V^T . P^T
+    // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------
 #pragma unroll
-    for (int db = 0; db < 8; db++) {
-      u32x4 a;
-      if (!FP8) {
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vl + va[db]));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vl + 4096 + va[db]));
-        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-        a = u32x4{l2[0], l2[1], h2[0], h2[1]};
-      } else {
-        i32x2 r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vl + va[db]));
-        a = widen8<QT>((uint32_t)r[0], (uint32_t)r[1]);
-      }
+    for (int db = 0; db < 8; db++)
 #pragma unroll
-      for (int rb = 0; rb < NRB; rb++) o_acc[rb][db] = Mma<QT>::run(a, pk[rb], o_acc[rb][db]);
-    }
+      for (int rb = 0; rb < NRB; rb++) o_acc[rb][db] = Mma<QT>::run(va_op[db], pk[rb], o_acc[rb][db]);
   };
 
-  auto end_segment = [&](const Cursor& cu, bool complete, int which) {
+  auto end_segment = [&](const Cursor& cu, bool complete, int which) __attribute__((always_inline)) {
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       int r = rg * (16 * NRB) + rb * 16 + c;
@@ -501,19 +569,20 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
     }
   };
 
-  // ---- software pipeline over this wave's tiles ---------------------------------------------------------
+  // ---- software pipeline over this wave's tiles: stage u lives in LDS slot u % NS -------------------------
   Cursor ci = start, cc = start;
   int issued = 0;
   for (; issued < NS - 1 && issued < n_units; ++issued) {
-    issue(ci, issued % NS);
-    cursor_next<PS16>(ci, p.seqlens, p.batch, p.page_size);
+    issue(ci, issued);
+    cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
   }
   bool seg_open = false;
   int seg_first_j = 0, seg_count = 0;
-  for (int u = 0; u < n_units; ++u) {
+  auto stage = [&](auto slot_c, int u) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value;
     if (issued < n_units) {
-      issue(ci, issued % NS);
-      cursor_next<PS16>(ci, p.seqlens, p.batch, p.page_size);
+      issue(ci, (SLOT + NS - 1) % NS);
+      cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
       ++issued;
     }
     if (!seg_open) {
@@ -526,14 +595,20 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
     else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * G::IPS>();
     else if (ahead == 1) wait_vmcnt<G::IPS>();
     else wait_vmcnt<0>();
-    compute(cc, u % NS);
+    compute(slot_c, cc);
     const bool last_of_seq = cc.j == cc.nt - 1;
     if (last_of_seq || u == n_units - 1) {
       end_segment(cc, seg_first_j == 0 && last_of_seq, seg_count == 0 ? 0 : 1);
       seg_open = false;
       ++seg_count;
     }
-    cursor_next<PS16>(cc, p.seqlens, p.batch, p.page_size);
+    cursor_next(cc, p.seqlens, p.batch, p.page_size, ps16);
+  };
+  for (int u = 0; u < n_units; u += NS) {
+    stage(IntC<0>{}, u);
+    if (NS > 1 && u + 1 < n_units) stage(IntC<1 % NS>{}, u + 1);
+    if (NS > 2 && u + 2 < n_units) stage(IntC<2 % NS>{}, u + 2);
+    if (NS > 3 && u + 3 < n_units) stage(IntC<3 % NS>{}, u + 3);
   }
 }
 
@@ -569,7 +644,7 @@ __global__ __launch_bounds__(kD) void paged_decode_mfma_combine_kernel(const Dec
     for (int pp = p_first; pp <= p_last; pp++) {
       if (!owns_tiles(pp)) continue;
       int64_t sl = slot_of(pp);
-      float w = exp2f(p.part_lse[sl] - M);
+      float w = fast_exp2(p.part_lse[sl] - M);
       W += w;
       A += w * p.part_o[sl * kD + d];
     }
@@ -586,19 +661,10 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   const int grid = (int)((waves + kNW - 1) / kNW);
   const size_t lds = (size_t)kNW * NS * Geom<KVT>::STAGE;
-  const bool ps16 = p.page_size == 16, cap = p.softcap > 0.f;
-#define MI355_LAUNCH(SC, P16)                                                                                         \
-  do {                                                                                                                \
-    auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, SC, P16>;                                                  \
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
-    if (e != hipSuccess) return hipGetErrorString(e);                                                                 \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);                                       \
-  } while (0)
-  if (cap && ps16) MI355_LAUNCH(true, true);
-  else if (cap) MI355_LAUNCH(true, false);
-  else if (ps16) MI355_LAUNCH(false, true);
-  else MI355_LAUNCH(false, false);
-#undef MI355_LAUNCH
+  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS>;
+  hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e0 != hipSuccess) return hipGetErrorString(e0);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
   hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(kD), 0, s, p, ws_prefix);
