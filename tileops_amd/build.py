@@ -40,9 +40,9 @@ def _hipcc() -> str:
     return exe
 
 
-def _compile(src: str) -> Path:
-    obj = OBJ_DIR / (src + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+def _compile(src: str, extra: tuple = (), tag: str = "") -> Path:
+    obj = OBJ_DIR / (src + tag + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stderr}")
@@ -54,20 +54,22 @@ def _compile(src: str) -> Path:
     return obj
 
 
-def build(verbose: bool = True) -> Path:
+def build(verbose: bool = True, extra_flags: tuple = (), lib_path: Path = LIB_PATH) -> Path:
+    """Compile and link.  ``extra_flags`` / ``lib_path`` let a developer build an instrumented copy beside the product."""
     OBJ_DIR.mkdir(exist_ok=True)
-    LIB_DIR.mkdir(exist_ok=True)
+    lib_path.parent.mkdir(exist_ok=True)
+    tag = "" if not extra_flags else "." + lib_path.stem
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
-        objs = list(pool.map(_compile, SOURCES))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
+        objs = list(pool.map(lambda src: _compile(src, tuple(extra_flags), tag), SOURCES))
+    tmp = lib_path.with_suffix(".so.tmp")
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
     if verbose:
-        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
-    return LIB_PATH
+        print(f"built {lib_path} ({lib_path.stat().st_size} bytes)")
+    return lib_path
 
 
 if __name__ == "__main__":

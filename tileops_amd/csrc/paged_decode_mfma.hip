@@ -107,6 +107,9 @@ __device__ __forceinline__ const char* uni_ptr(const char* p) {
 // LDS-DMA wait state and the five wait states a VMEM instruction needs after a VALU write of its SGPR base,
 // which the compiler's hazard recogniser cannot insert inside an asm block.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const char* sbase) {
+#ifdef MI355_DEBUG_NO_DMA
+  return;
+#endif
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   sbase = uni_ptr(sbase);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
@@ -211,7 +214,9 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
     T += n;
   }
   T = uni(T);
-  if (gw == 0) {  // exclusive prefix of tiles per sequence, for the combine kernel
+  if (gw == 0) {
+    // Per-sequence record for the combine kernel: {first tile, first partition, last partition, whether the
+    // first partition holds this sequence in its second partial slot}.  Entry [batch] = {T, 0, 0, 0}.
     int carry = 0;
     for (int base = 0; base < p.batch; base += 64) {
       int b = base + lane;
@@ -222,10 +227,19 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
         int t = __shfl_up(incl, d, 64);
         if (lane >= d) incl += t;
       }
-      if (b < p.batch) ws_prefix[b] = carry + incl - n;
+      if (b < p.batch) {
+        int pre = carry + incl - n;
+        int4 rec = {pre, 0, 0, 0};
+        if (n > 0) {
+          rec.y = part_of(pre, T, NP);
+          rec.z = part_of(pre + n - 1, T, NP);
+          rec.w = part_begin(rec.y, T, NP) != pre ? 1 : 0;
+        }
+        ((int4*)ws_prefix)[b] = rec;
+      }
       carry += __shfl(incl, 63, 64);
     }
-    if (lane == 0) ws_prefix[p.batch] = T;
+    if (lane == 0) ((int4*)ws_prefix)[p.batch] = int4{T, 0, 0, 0};
   }
   if (part >= p.n_parts || T == 0) return;
   const int u0 = part_begin(part, T, NP), u1 = part_begin(part + 1, T, NP);
@@ -461,6 +475,14 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
       for (int db = 0; db < 8; db++) va_op[db] = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
     }
     if (!FP8) __builtin_amdgcn_sched_barrier(0);
+#ifdef MI355_ABL_NO_LDS
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) ka_op[tb][j] = qreg[0][j];
+#pragma unroll
+    for (int db = 0; db < 8; db++) va_op[db] = qreg[0][db & 3];
+#endif
     // ---- S^T = K . Q^T : the two 16-token blocks interleaved so dependent MFMAs are one apart -------------
     f32x4 s_acc[2][NRB];
 #pragma unroll
@@ -472,7 +494,13 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-        for (int tb = 0; tb < 2; tb++) s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
+        for (int tb = 0; tb < 2; tb++) {
+#ifndef MI355_ABL_NO_QK
+          s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
+#else
+          s_acc[tb][rb][j] += __uint_as_float(ka_op[tb][j][0]);
+#endif
+        }
     // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
     const bool need_mask = tok0 + kCT > cu.len - qoff;
     u32x4 pk[NRB];
@@ -507,6 +535,12 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
           for (int i = 0; i < 4; i++)
             if (tok0 + 16 * tb + 4 * g + i >= limit[rb]) x[tb][i] = -INFINITY;
       }
+#ifdef MI355_ABL_NO_SOFTMAX
+      alpha[rb] = 1.f;
+      pk[rb][0] = __float_as_uint(x[0][0]); pk[rb][1] = __float_as_uint(x[0][2]); pk[rb][2] = __float_as_uint(x[1][0]); pk[rb][3] = __float_as_uint(x[1][3]);
+      l_run[rb] += x[0][1];
+      continue;
+#endif
       float mt = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])), fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
       mt = group_max(mt);
       float m_new = fmaxf(m_run[rb], mt);
@@ -538,7 +572,13 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 #pragma unroll
     for (int db = 0; db < 8; db++)
 #pragma unroll
-      for (int rb = 0; rb < NRB; rb++) o_acc[rb][db] = Mma<QT>::run(va_op[db], pk[rb], o_acc[rb][db]);
+      for (int rb = 0; rb < NRB; rb++) {
+#ifndef MI355_ABL_NO_PV
+        o_acc[rb][db] = Mma<QT>::run(va_op[db], pk[rb], o_acc[rb][db]);
+#else
+        o_acc[rb][db][0] += __uint_as_float(va_op[db][0] ^ pk[rb][0]);
+#endif
+      }
   };
 
   auto end_segment = [&](const Cursor& cu, bool complete, int which) __attribute__((always_inline)) {
@@ -595,7 +635,9 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
     else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * G::IPS>();
     else if (ahead == 1) wait_vmcnt<G::IPS>();
     else wait_vmcnt<0>();
+#ifndef MI355_DEBUG_NO_COMPUTE
     compute(slot_c, cc);
+#endif
     const bool last_of_seq = cc.j == cc.nt - 1;
     if (last_of_seq || u == n_units - 1) {
       end_segment(cc, seg_first_j == 0 && last_of_seq, seg_count == 0 ? 0 : 1);
@@ -613,46 +655,67 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
 }
 
 // Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
-// grid (heads_kv*rows, batch), 128 threads (one per head element).
+//   lse = log2 sum_s 2^(lse_s - max) + max ; O = sum_s 2^(lse_s - lse) * O_s   (reference combine,
+//   src/tileops/kernels/attention/gqa_decode_paged.py:344-374), on fp32 partials.
+// One wave per (sequence, kv head, query row): lane i fetches the LSE of the i-th partition of the sequence,
+// the weights are formed with two wave reductions, then every lane accumulates two head elements over the
+// partitions with independent loads.  grid (heads_kv*rows, batch), 64 threads.
 template <typename QT>
-__global__ __launch_bounds__(kD) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix) {
-  const int b = blockIdx.y, row_all = blockIdx.x, d = threadIdx.x;
+__global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix) {
+  const int b = blockIdx.y, row_all = blockIdx.x, lane = threadIdx.x;
   const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
   const int s = r / p.group, gi = r - s * p.group;
-  uint16_t* op = (uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD + d;
-  const int len = p.seqlens[b];
-  const int nt = units_of(len);
-  if (nt == 0) {
+  uint32_t* op = (uint32_t*)((uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) + lane;
+  if (p.seqlens[b] <= 0) {
     *op = 0;
     return;
   }
-  const int64_t T = ws_prefix[p.batch], NP = p.n_parts, pre = ws_prefix[b];
-  const int p_first = part_of(pre, T, NP), p_last = part_of(pre + nt - 1, T, NP);
+  const int4 rec = ((const int4*)ws_prefix)[b];
+  const int p_first = rec.y, p_last = rec.z;
   if (p_first == p_last) return;  // one wave covered the whole sequence and wrote the output itself
+  const int64_t T = ((const int4*)ws_prefix)[p.batch].x, NP = p.n_parts;
+  const bool gaps = T < NP;  // fewer tiles than partitions: partitions in between may own nothing
   const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
-  auto slot_of = [&](int pp) -> int64_t {
-    int which = (pp == p_first && part_begin(pp, T, NP) != pre) ? 1 : 0;
-    return (int64_t)(2 * pp + which) * rows_all + row_all;
-  };
-  // with fewer tiles than partitions some partitions in between own no tile and wrote nothing
-  auto owns_tiles = [&](int pp) { return part_begin(pp + 1, T, NP) > part_begin(pp, T, NP); };
-  float M = -INFINITY;
-  for (int pp = p_first; pp <= p_last; pp++)
-    if (owns_tiles(pp)) M = fmaxf(M, p.part_lse[slot_of(pp)]);
-  float W = 0.f, A = 0.f;
-  if (M > -INFINITY) {
-    for (int pp = p_first; pp <= p_last; pp++) {
-      if (!owns_tiles(pp)) continue;
-      int64_t sl = slot_of(pp);
-      float w = fast_exp2(p.part_lse[sl] - M);
-      W += w;
-      A += w * p.part_o[sl * kD + d];
+  const int n = p_last - p_first + 1;
+  float acc0 = 0.f, acc1 = 0.f, W = 0.f, M = -INFINITY;
+  for (int base = 0; base < n; base += 64) {  // a sequence seldom spans more than a handful of partitions
+    const int pp = p_first + base + lane;
+    bool valid = pp <= p_last;
+    if (valid && gaps) valid = part_begin(pp + 1, T, NP) > part_begin(pp, T, NP);
+    const int64_t slot = (int64_t)(2 * pp + ((pp == p_first && rec.w) ? 1 : 0)) * rows_all + row_all;
+    const float lse = valid ? p.part_lse[slot] : -INFINITY;
+    float m_chunk = lse;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) m_chunk = fmaxf(m_chunk, __shfl_xor(m_chunk, m, 64));
+    const float M_new = fmaxf(M, m_chunk);
+    if (M_new == -INFINITY) continue;
+    const float rescale = fast_exp2(M - M_new);  // 0 on the first chunk (M = -inf)
+    acc0 *= rescale;
+    acc1 *= rescale;
+    W *= rescale;
+    M = M_new;
+    const float w_lane = valid ? fast_exp2(lse - M) : 0.f;
+    float w_sum = w_lane;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) w_sum += __shfl_xor(w_sum, m, 64);
+    W += w_sum;
+    const int cnt = min(64, n - base);
+#pragma unroll 4
+    for (int i = 0; i < cnt; i++) {
+      const float w = __shfl(w_lane, i, 64);
+      const int64_t sl = __shfl(slot, i, 64);
+      if (w != 0.f) {
+        const f32x2 v = *(const f32x2*)(p.part_o + sl * kD + 2 * lane);
+        acc0 = fmaf(w, v[0], acc0);
+        acc1 = fmaf(w, v[1], acc1);
+      }
     }
   }
-  *op = f32_to_elem_bits<QT>(W > 0.f ? A / W : 0.f);
+  const float inv = W > 0.f ? 1.0f / W : 0.f;
+  *op = Mma<QT>::pack(acc0 * inv, acc1 * inv);
 }
 
-template <typename KVT> constexpr int stages_for() { return Geom<KVT>::FP8 ? 3 : 2; }
+template <typename KVT> constexpr int stages_for() { return 2; }
 
 template <typename QT, typename KVT, int NRB>
 const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
@@ -667,7 +730,7 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
-  hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(kD), 0, s, p, ws_prefix);
+  hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
@@ -700,16 +763,16 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
   const int nrb = row_blocks_for(rows);
   const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
-  const int wgs_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 1 : 1;
+  const int wgs_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 2 : 1;
   const int64_t waves = (int64_t)kNumCU * wgs_per_cu * kNW;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
 }
 
-// [part_o: 2*n_parts slots x heads_kv*rows x dim fp32][part_lse: 2*n_parts x heads_kv*rows fp32][prefix: batch+1 int32]
+// [part_o: 2*n_parts slots x heads_kv*rows x dim fp32][part_lse: 2*n_parts x heads_kv*rows fp32][records: (batch+1) x int4]
 size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int batch) {
   size_t slots = (size_t)2 * n_parts * heads_kv * rows;
-  return align256(slots * dim * sizeof(float)) + align256(slots * sizeof(float)) + align256((size_t)(batch + 1) * sizeof(int));
+  return align256(slots * dim * sizeof(float)) + align256(slots * sizeof(float)) + align256((size_t)(batch + 1) * 4 * sizeof(int));
 }
 
 const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, hipStream_t s) {
