@@ -193,6 +193,8 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
   const int lane = threadIdx.x & 63;
   const int c = lane & 15, g = lane >> 4;
   const int wave = uni(threadIdx.x >> 6);
+  // Workgroups are dealt round-robin to the 8 XCDs, so neighbouring partitions (which read neighbouring pages of
+  // a sequence) spread over all L2s and memory channels; renumbering them XCD-contiguously measured slower.
   const int gw = blockIdx.x * kNW + wave;
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int per_part = p.heads_kv * n_rg;
@@ -229,11 +231,11 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
       }
       if (b < p.batch) {
         int pre = carry + incl - n;
-        int4 rec = {pre, 0, 0, 0};
+        int4 rec = {pre, -1, -1, 0};  // y < 0 marks an empty sequence
         if (n > 0) {
           rec.y = part_of(pre, T, NP);
           rec.z = part_of(pre + n - 1, T, NP);
-          rec.w = part_begin(rec.y, T, NP) != pre ? 1 : 0;
+          rec.w = (part_begin(rec.y, T, NP) != pre ? 1 : 0) | (T < NP ? 2 : 0);  // bit 1: some partitions own no tile
         }
         ((int4*)ws_prefix)[b] = rec;
       }
@@ -666,24 +668,33 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
   const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
   const int s = r / p.group, gi = r - s * p.group;
   uint32_t* op = (uint32_t*)((uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) + lane;
-  if (p.seqlens[b] <= 0) {
+  const int4 rec = ((const int4*)ws_prefix)[b];  // the only load everything else depends on
+  const int p_first = rec.y, p_last = rec.z;
+  if (p_first < 0) {  // empty sequence: the attention kernel never visits it
     *op = 0;
     return;
   }
-  const int4 rec = ((const int4*)ws_prefix)[b];
-  const int p_first = rec.y, p_last = rec.z;
   if (p_first == p_last) return;  // one wave covered the whole sequence and wrote the output itself
-  const int64_t T = ((const int4*)ws_prefix)[p.batch].x, NP = p.n_parts;
-  const bool gaps = T < NP;  // fewer tiles than partitions: partitions in between may own nothing
+  const bool gaps = (rec.w & 2) != 0, first_in_slot1 = (rec.w & 1) != 0;
+  const int64_t NP = p.n_parts;
+  const int64_t T = gaps ? ((const int4*)ws_prefix)[p.batch].x : 0;
   const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
   const int n = p_last - p_first + 1;
+  auto slot_of = [&](int pp) { return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all; };
   float acc0 = 0.f, acc1 = 0.f, W = 0.f, M = -INFINITY;
   for (int base = 0; base < n; base += 64) {  // a sequence seldom spans more than a handful of partitions
     const int pp = p_first + base + lane;
     bool valid = pp <= p_last;
     if (valid && gaps) valid = part_begin(pp + 1, T, NP) > part_begin(pp, T, NP);
-    const int64_t slot = (int64_t)(2 * pp + ((pp == p_first && rec.w) ? 1 : 0)) * rows_all + row_all;
-    const float lse = valid ? p.part_lse[slot] : -INFINITY;
+    const float lse = valid ? p.part_lse[slot_of(pp)] : -INFINITY;
+    // the first eight partials are fetched together with the LSEs, before the weights are known
+    constexpr int PRE = 8;
+    f32x2 pre_v[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+      const int pi = min(p_first + base + i, p_last);
+      pre_v[i] = *(const f32x2*)(p.part_o + slot_of(pi) * kD + 2 * lane);
+    }
     float m_chunk = lse;
 #pragma unroll
     for (int m = 1; m < 64; m <<= 1) m_chunk = fmaxf(m_chunk, __shfl_xor(m_chunk, m, 64));
@@ -700,12 +711,18 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
     for (int m = 1; m < 64; m <<= 1) w_sum += __shfl_xor(w_sum, m, 64);
     W += w_sum;
     const int cnt = min(64, n - base);
-#pragma unroll 4
-    for (int i = 0; i < cnt; i++) {
-      const float w = __shfl(w_lane, i, 64);
-      const int64_t sl = __shfl(slot, i, 64);
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+      const float w = __shfl(w_lane, i, 64);  // 0 for lanes past the last partition
       if (w != 0.f) {
-        const f32x2 v = *(const f32x2*)(p.part_o + sl * kD + 2 * lane);
+        acc0 = fmaf(w, pre_v[i][0], acc0);
+        acc1 = fmaf(w, pre_v[i][1], acc1);
+      }
+    }
+    for (int i = PRE; i < cnt; i++) {
+      const float w = __shfl(w_lane, i, 64);
+      if (w != 0.f) {
+        const f32x2 v = *(const f32x2*)(p.part_o + slot_of(p_first + base + i) * kD + 2 * lane);
         acc0 = fmaf(w, v[0], acc0);
         acc1 = fmaf(w, v[1], acc1);
       }
