@@ -42,8 +42,11 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     if kernel_key:
         op.kernel_map = {kernel_key: op.kernel_map[kernel_key]}
     args = inp.as_args()
-    # 512 MiB scratch written between steps evicts L2 and the 256 MB Infinity Cache, so every step reads HBM
+    # Between steps a 512 MiB buffer is overwritten and a second 512 MiB buffer is read: the write evicts L2 and
+    # the 256 MB Infinity Cache, the read pushes the dirty lines out again so the timed call starts on a clean,
+    # cold cache and every K/V byte comes from HBM.
     flush = torch.empty(512 << 20, dtype=torch.uint8, device=device)
+    flush_rd = torch.ones(128 << 20, dtype=torch.int32, device=device)
     for _ in range(max(warmup, 1)):
         out = op(*args)
     torch.cuda.synchronize()
@@ -54,6 +57,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     wall0 = time.perf_counter()
     for i in range(steps):
         flush.fill_(i & 0xFF)
+        flush_rd.max()
         starts[i].record()
         out = op(*args)
         stops[i].record()
@@ -70,6 +74,26 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     torch.cuda.synchronize()
     b2b_ms = s0.elapsed_time(s1) / steps
 
+    # The dominant (attention) kernel alone: launches that skip the combine kernel, KREP back to back per event
+    # pair so that the few microseconds an event pair costs are spread over KREP launches.  Each launch streams
+    # far more than the 256 MB Infinity Cache holds, so a launch finds next to nothing of its predecessor cached.
+    KREP = 4
+    kernel = next(iter(next(iter(op._kernel_roles.values())).values()))
+    kernel.attention_kernel_only = True
+    k_starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    k_stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        flush.fill_(i & 0xFF)
+        flush_rd.max()
+        k_starts[i].record()
+        for _ in range(KREP):
+            op(*args)
+        k_stops[i].record()
+    torch.cuda.synchronize()
+    kernel.attention_kernel_only = False
+    kernel_ms = sum(s.elapsed_time(e) for s, e in zip(k_starts, k_stops)) / (steps * KREP)
+    out = op(*args)  # complete output again for the parity check below
+
     lens = inp.real_seqlen_kv.cpu().to(torch.int64)
     sum_len = int(lens.sum())
     sum_pages = int(((lens + cfg.page_size - 1) // cfg.page_size).sum())
@@ -77,8 +101,12 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     b = algorithmic_bytes(sum_len=sum_len, sum_pages=sum_pages, batch=cfg.batch, q_len=cfg.q_len, heads=cfg.heads, heads_kv=cfg.heads_kv,
                           dim=cfg.dim, q_bytes=2, kv_bytes=1 if fp8 else 2, fp8_scales=fp8)
     flops = algorithmic_flops(sum_len=sum_len, q_len=cfg.q_len, heads=cfg.heads, dim=cfg.dim)
-    achieved = b["total"] / (ms * 1e-3) / 1e9
-    kernel = next(iter(next(iter(op._kernel_roles.values())).values()))
+    achieved = b["total"] / (kernel_ms * 1e-3) / 1e9
+    traffic = None
+    try:  # measured with hardware counters in a separate profiler run; absent for configurations not profiled
+        traffic = json.loads((ROOT / "profiles" / "hbm_traffic.json").read_text()).get(name, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        pass
     res = {
         "workload": f"{name}: {cfg.description}; batch {cfg.batch}, q_len {cfg.q_len}, {cfg.heads}q/{cfg.heads_kv}kv heads, dim {cfg.dim}, "
                     f"page {cfg.page_size}, len in {list(cfg.len_range)}, {cfg.n_pages}-page pool, seed {cfg.seed}",
@@ -92,8 +120,12 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         "algorithmic_bytes": b,
         "flops": flops,
         "kv_read_gbs": (b["kv"] + b["scales"]) / (ms * 1e-3) / 1e9,
+        "attention_kernel_us": kernel_ms * 1e3,
+        "whole_call_gbs": b["total"] / (ms * 1e-3) / 1e9,
+        "whole_call_frac_of_peak": b["total"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        # dominant kernel: algorithmic bytes of one launch / its own duration (events around the attention kernel alone)
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None},
+                     "traffic": traffic},
         "wall_s_timed_region": wall,
     }
     if with_cpu:
@@ -122,7 +154,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
                                "sample": f"torch fp32 oracle on the first {n_seq} of {cfg.batch} sequences ({sample_len} of {sum_len} KV tokens), "
                                          f"median of 3 runs, scaled by tokens to the whole batch"}
         res["parity"] = {"max_abs_err": err, "tolerance": tol, "within_tolerance": bool(ok), "sequences_checked": n_seq}
-    del inp, args, flush
+    del inp, args, flush, flush_rd
     torch.cuda.empty_cache()
     return res
 
@@ -136,6 +168,8 @@ def main() -> None:
     ap.add_argument("--also", default="c3", help="comma-separated extra configurations reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
     ap.add_argument("--kernel", default=None, choices=[None, "gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel"])
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 1 GiB device copies, so a hardware-counter pass has a kernel of known traffic to scale by")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the path is single-GPU by construction (every (sequence, kv-head) is independent); "
@@ -161,6 +195,13 @@ def main() -> None:
         line["parity"] = main_res["parity"]
     line["detail"] = {k: v for k, v in main_res.items() if k not in ("roofline", "cpu_baseline", "parity", "workload")}
     line["also"] = also
+    if a.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["copy_calibration"] = {"bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "launches": 3}
     print(json.dumps(line))
 
 

@@ -104,8 +104,8 @@ int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_
   if (rc) return rc;
   Plan plan;
   // softcap does not change the plan; the MFMA kernel serves both settings
-  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in, kernel,
-                 &plan);
+  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in,
+                 kernel & ~MI355_KERNEL_FLAG_SKIP_COMBINE, &plan);
   if (rc) return rc;
   if (workspace_bytes) *workspace_bytes = plan.part_o_bytes + plan.part_lse_bytes;
   if (num_split_out) *num_split_out = plan.kernel == MI355_KERNEL_GENERIC ? plan.max_splits : plan.n_parts;
@@ -120,6 +120,8 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
                            int num_split, int kernel, void* hip_stream) {
   int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
   if (rc) return rc;
+  const bool skip_combine = (kernel & MI355_KERNEL_FLAG_SKIP_COMBINE) != 0;
+  kernel &= ~MI355_KERNEL_FLAG_SKIP_COMBINE;
   if (batch == 0) return MI355_OK;
   if (!q || !k || !v || !seqlens || !block_table || !out)
     return fail(MI355_EINVAL, "q, k, v, seqlens, block_table and out must be non-null");
@@ -183,9 +185,9 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
   const char* err;
   if (plan.kernel == MI355_KERNEL_GENERIC) {
     err = launch_generic(p, q_dtype, kv_dtype, s);
-    if (!err) err = launch_generic_combine(p, q_dtype, s);
+    if (!err && !skip_combine) err = launch_generic_combine(p, q_dtype, s);
   } else {
-    err = launch_mfma(p, q_dtype, kv_dtype, s);
+    err = launch_mfma(p, q_dtype, kv_dtype, skip_combine, s);
   }
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
   return MI355_OK;

@@ -735,18 +735,26 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
 template <typename KVT> constexpr int stages_for() { return 2; }
 
 template <typename QT, typename KVT, int NRB>
-const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
+const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   constexpr int NS = stages_for<KVT>();
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   const int grid = (int)((waves + kNW - 1) / kNW);
   const size_t lds = (size_t)kNW * NS * Geom<KVT>::STAGE;
   auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS>;
-  hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e0 != hipSuccess) return hipGetErrorString(e0);
+  // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
+  static bool lds_opted_in[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return "hipGetDevice failed";
+  if (dev < 0 || dev >= 64 || !lds_opted_in[dev]) {
+    hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e0 != hipSuccess) return hipGetErrorString(e0);
+    if (dev >= 0 && dev < 64) lds_opted_in[dev] = true;
+  }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
+  if (skip_combine) return nullptr;
   hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
@@ -755,11 +763,11 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
 int row_blocks_for(int rows) { return rows <= 16 ? 1 : (rows <= 32 ? 2 : 4); }
 
 template <typename QT, typename KVT>
-const char* launch_t2(const DecodeParams& p, int* ws_prefix, hipStream_t s) {
+const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   switch (row_blocks_for(p.rows)) {
-    case 1: return launch_t3<QT, KVT, 1>(p, ws_prefix, s);
-    case 2: return launch_t3<QT, KVT, 2>(p, ws_prefix, s);
-    default: return launch_t3<QT, KVT, 4>(p, ws_prefix, s);
+    case 1: return launch_t3<QT, KVT, 1>(p, ws_prefix, skip_combine, s);
+    case 2: return launch_t3<QT, KVT, 2>(p, ws_prefix, skip_combine, s);
+    default: return launch_t3<QT, KVT, 4>(p, ws_prefix, skip_combine, s);
   }
 }
 
@@ -792,17 +800,17 @@ size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int ba
   return align256(slots * dim * sizeof(float)) + align256(slots * sizeof(float)) + align256((size_t)(batch + 1) * 4 * sizeof(int));
 }
 
-const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, hipStream_t s) {
+const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, bool skip_combine, hipStream_t s) {
   DecodeParams p = p_in;
   size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
   char* ws = (char*)p_in.part_o;
   p.part_o = (float*)ws;
   p.part_lse = (float*)(ws + align256(slots * kD * sizeof(float)));
   int* ws_prefix = (int*)(ws + align256(slots * kD * sizeof(float)) + align256(slots * sizeof(float)));
-  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag>(p, ws_prefix, s);
-  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag>(p, ws_prefix, s);
-  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag>(p, ws_prefix, s);
-  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag>(p, ws_prefix, s);
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag>(p, ws_prefix, skip_combine, s);
   return "MFMA kernel: unsupported (q_dtype, kv_dtype) pair";
 }
 

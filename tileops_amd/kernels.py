@@ -250,6 +250,10 @@ class GQADecodePagedKernel(Kernel):
             plan = self._plans[key] = (nbytes, nsplit)
         return plan
 
+    #: Measurement aid: when True, ``forward`` launches the attention kernel alone (no combine), so a benchmark
+    #: can time the dominant kernel by itself.  The returned tensor is then incomplete.
+    attention_kernel_only: bool = False
+
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor,
                 block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
                 v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -261,7 +265,8 @@ class GQADecodePagedKernel(Kernel):
             q, k, v, k_scale, v_scale, real_seqlen_kv, block_table, out, workspace,
             batch=self.batch, q_len=self.q_len, heads=self.heads, heads_kv=self.groups, dim=self.dim,
             page_size=self.page_size, sm_scale=self.sm_scale, softcap=self.softcap, causal=self.is_causal,
-            num_split=nsplit, kernel=self._native_kernel)
+            num_split=nsplit,
+            kernel=self._native_kernel | (native.KERNEL_FLAG_SKIP_COMBINE if self.attention_kernel_only else 0))
         return out
 
 
