@@ -43,7 +43,6 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // head dim served by this kernel
-constexpr int kNW = 4;        // waves per workgroup
 constexpr int kNumCU = 256;   // MI355X
 
 template <typename KVT> struct Geom {
@@ -184,8 +183,8 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict
 // ------------------------------------------------------------------------------------------------------
 template <int V> struct IntC { static constexpr int value = V; };
 
-template <typename QT, typename KVT, int NRB, int NS>
-__global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+template <typename QT, typename KVT, int NRB, int NS, int NW>
+__global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -195,7 +194,7 @@ __global__ __launch_bounds__(kNW * 64) void paged_decode_mfma_kernel(const Decod
   const int wave = uni(threadIdx.x >> 6);
   // Workgroups are dealt round-robin to the 8 XCDs, so neighbouring partitions (which read neighbouring pages of
   // a sequence) spread over all L2s and memory channels; renumbering them XCD-contiguously measured slower.
-  const int gw = blockIdx.x * kNW + wave;
+  const int gw = blockIdx.x * NW + wave;
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int per_part = p.heads_kv * n_rg;
   // integer division runs on the vector ALU; pin the results to scalar registers so that everything derived
@@ -732,16 +731,19 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
   *op = Mma<QT>::pack(acc0 * inv, acc1 * inv);
 }
 
-template <typename KVT> constexpr int stages_for() { return 2; }
+// Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
+// fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
+// 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
+template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB == 1) ? 8 : 4; }
 
 template <typename QT, typename KVT, int NRB>
 const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  constexpr int NS = stages_for<KVT>();
+  constexpr int NS = 2, NW = waves_per_wg<KVT, NRB>();
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
-  const int grid = (int)((waves + kNW - 1) / kNW);
-  const size_t lds = (size_t)kNW * NS * Geom<KVT>::STAGE;
-  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS>;
+  const int grid = (int)((waves + NW - 1) / NW);
+  const size_t lds = (size_t)NW * NS * Geom<KVT>::STAGE;
+  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
   static bool lds_opted_in[64] = {};
   int dev = 0;
@@ -751,7 +753,7 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
     if (e0 != hipSuccess) return hipGetErrorString(e0);
     if (dev >= 0 && dev < 64) lds_opted_in[dev] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kNW * 64), lds, s, p, ws_prefix);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, s, p, ws_prefix);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
   if (skip_combine) return nullptr;
@@ -788,8 +790,8 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
   const int nrb = row_blocks_for(rows);
   const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
-  const int wgs_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 2 : 1;
-  const int64_t waves = (int64_t)kNumCU * wgs_per_cu * kNW;
+  const int waves_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 8 : 4;  // what the LDS of a CU holds, two stages per wave
+  const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
 }
