@@ -44,6 +44,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
+constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
   static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
@@ -181,8 +182,6 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------------
-template <int V> struct IntC { static constexpr int value = V; };
-
 template <typename QT, typename KVT, int NRB, int NS, int NW>
 __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
@@ -432,8 +431,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       for (int j = 0; j < 4; j++) asm volatile("" : "+v"(qreg[rb][j]));
   };
 
-  auto compute = [&](auto slot_c, const Cursor& cu) __attribute__((always_inline)) {
-    constexpr int SOFF = decltype(slot_c)::value * G::STAGE;
+  // SOFF = byte offset of the stage slot inside the wave's LDS ring; a literal at every call site of the
+  // single-row-block kernels (folds into the ds_read immediates), a run-time value in the multi-row-block ones
+  auto compute = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
     u32x4 ka_op[2][4], va_op[8];
@@ -506,7 +506,6 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     const bool need_mask = tok0 + kCT > cu.len - qoff;
     u32x4 pk[NRB];
     float alpha[NRB];
-    bool any_rescale = false;
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       float x[2][4];
@@ -544,8 +543,13 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
 #endif
       float mt = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])), fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
       mt = group_max(mt);
-      float m_new = fmaxf(m_run[rb], mt);
-      alpha[rb] = fast_exp2(m_run[rb] - m_new);
+      // Lazy rescale: the running reference m_run only moves when the tile maximum exceeds it by more than
+      // kRescaleGap (log2 domain).  Probabilities are then at most 2^kRescaleGap instead of 1 -- harmless for
+      // fp32 accumulators and 16-bit P -- and because l_run uses the same reference the final O/l is unchanged.
+      // After the first tiles of a sequence the accumulator rescale below almost never runs.
+      const bool moved = mt > m_run[rb] + kRescaleGap;
+      const float m_new = moved ? mt : m_run[rb];
+      alpha[rb] = moved ? fast_exp2(m_run[rb] - m_new) : 1.0f;
       m_run[rb] = m_new;
       float psum = 0.f;
 #pragma unroll
@@ -561,13 +565,17 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       pk[rb][1] = Mma<QT>::pack(x[0][2], x[0][3]);
       pk[rb][2] = Mma<QT>::pack(x[1][0], x[1][1]);
       pk[rb][3] = Mma<QT>::pack(x[1][2], x[1][3]);
-      any_rescale |= alpha[rb] != 1.0f;
-    }
-    if (__any(any_rescale)) {
+      if (__builtin_expect(__any(moved), 0)) {  // wave-uniform: some row of this row block moved its reference
+        // The accumulators live in accumulation registers, which the vector ALU cannot address: the two empty
+        // asm statements pin them there on entry and exit, so the copies out and back stay inside this rarely
+        // taken block instead of being hoisted into every loop iteration.
 #pragma unroll
-      for (int rb = 0; rb < NRB; rb++)
-#pragma unroll
-        for (int db = 0; db < 8; db++) o_acc[rb][db] *= alpha[rb];
+        for (int db = 0; db < 8; db++) {
+          asm volatile("" : "+a"(o_acc[rb][db]));
+          o_acc[rb][db] *= alpha[rb];
+          asm volatile("" : "+a"(o_acc[rb][db]));
+        }
+      }
     }
     // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------
 #pragma unroll
@@ -611,47 +619,60 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   };
 
   // ---- software pipeline over this wave's tiles: stage u lives in LDS slot u % NS -------------------------
+  // Outer loop = segments (maximal runs of tiles of one sequence inside this wave's range), inner loop = the
+  // tiles of a segment.  The accumulators are initialised in the inner loop's preheader and stay in their
+  // registers across it; issuing runs NS-1 tiles ahead of consumption and is oblivious to segment borders.
   Cursor ci = start, cc = start;
   int issued = 0;
   for (; issued < NS - 1 && issued < n_units; ++issued) {
     issue(ci, issued);
     cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
   }
-  bool seg_open = false;
-  int seg_first_j = 0, seg_count = 0;
-  auto stage = [&](auto slot_c, int u) __attribute__((always_inline)) {
-    constexpr int SLOT = decltype(slot_c)::value;
+  auto issue_ahead = [&](int ring) __attribute__((always_inline)) {
     if (issued < n_units) {
-      issue(ci, (SLOT + NS - 1) % NS);
+      issue(ci, ring == 0 ? NS - 1 : ring - 1);  // the ring slot consumed in the previous iteration
       cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
       ++issued;
     }
-    if (!seg_open) {
-      begin_segment(cc);
-      seg_open = true;
-      seg_first_j = cc.j;
-    }
+  };
+  auto wait_stage = [&](int u) __attribute__((always_inline)) {
     const int ahead = issued - u - 1;  // stages issued after the one consumed now
     if (ahead >= 3) wait_vmcnt<(NS > 3 ? 3 : NS - 1) * G::IPS>();
     else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * G::IPS>();
     else if (ahead == 1) wait_vmcnt<G::IPS>();
     else wait_vmcnt<0>();
-#ifndef MI355_DEBUG_NO_COMPUTE
-    compute(slot_c, cc);
-#endif
-    const bool last_of_seq = cc.j == cc.nt - 1;
-    if (last_of_seq || u == n_units - 1) {
-      end_segment(cc, seg_first_j == 0 && last_of_seq, seg_count == 0 ? 0 : 1);
-      seg_open = false;
-      ++seg_count;
-    }
-    cursor_next(cc, p.seqlens, p.batch, p.page_size, ps16);
   };
-  for (int u = 0; u < n_units; u += NS) {
-    stage(IntC<0>{}, u);
-    if (NS > 1 && u + 1 < n_units) stage(IntC<1 % NS>{}, u + 1);
-    if (NS > 2 && u + 2 < n_units) stage(IntC<2 % NS>{}, u + 2);
-    if (NS > 3 && u + 3 < n_units) stage(IntC<3 % NS>{}, u + 3);
+  auto run_compute = [&](int ring) __attribute__((always_inline)) {
+#ifndef MI355_DEBUG_NO_COMPUTE
+    if constexpr (NRB == 1) {
+      // one copy of the stage body per ring slot: the slot offset folds into the LDS read immediates
+      if (ring == 0) compute(0u, cc);
+      else if (NS > 1 && ring == 1) compute((uint32_t)G::STAGE, cc);
+      else if (NS > 2 && ring == 2) compute(2u * G::STAGE, cc);
+      else compute(3u * G::STAGE, cc);
+    } else {
+      compute((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
+    }
+#endif
+  };
+  int u = 0, ring = 0, seg_count = 0;
+  while (u < n_units) {
+    const int seg_first_j = cc.j;
+    const int seg_units = min(cc.nt - cc.j, n_units - u);
+    issue_ahead(ring);   // before the query loads, so the next tile is already in flight while they land
+    begin_segment(cc);
+    for (int k = 0; k < seg_units; ++k) {
+      if (k > 0) issue_ahead(ring);
+      wait_stage(u);
+      run_compute(ring);
+      ++u;
+      ++cc.j;
+      ring = ring + 1 == NS ? 0 : ring + 1;
+    }
+    --cc.j;  // end_segment and cursor_next see the last tile of the segment
+    end_segment(cc, seg_first_j == 0 && cc.j == cc.nt - 1, seg_count == 0 ? 0 : 1);
+    ++seg_count;
+    cursor_next(cc, p.seqlens, p.batch, p.page_size, ps16);
   }
 }
 
@@ -738,7 +759,8 @@ template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT
 
 template <typename QT, typename KVT, int NRB>
 const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  constexpr int NS = 2, NW = waves_per_wg<KVT, NRB>();
+  // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
+  constexpr int NS = (Geom<KVT>::FP8 && NRB > 1) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   const int grid = (int)((waves + NW - 1) / NW);
@@ -790,7 +812,9 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
   const int nrb = row_blocks_for(rows);
   const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
-  const int waves_per_cu = kv_dtype == MI355_DT_FP8_E4M3FN ? 8 : 4;  // what the LDS of a CU holds, two stages per wave
+  // resident waves per CU: eight for the fp8 single-row-block kernel (LDS-limited, ~160 VGPRs), otherwise four
+  // (LDS-limited with a 16-bit cache, register-limited -- one wave per SIMD -- with more than one row block)
+  const int waves_per_cu = (kv_dtype == MI355_DT_FP8_E4M3FN && nrb == 1) ? 8 : 4;
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
