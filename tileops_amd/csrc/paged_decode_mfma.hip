@@ -755,12 +755,12 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
 // Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
-template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB == 1) ? 8 : 4; }
+template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB <= 2) ? 8 : 4; }
 
 template <typename QT, typename KVT, int NRB>
 const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
-  constexpr int NS = (Geom<KVT>::FP8 && NRB > 1) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
+  constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   const int grid = (int)((waves + NW - 1) / NW);
@@ -784,11 +784,11 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
-int row_blocks_for(int rows) { return rows <= 16 ? 1 : (rows <= 32 ? 2 : 4); }
+int row_blocks_for(int rows, bool fp8) { return rows <= 16 ? 1 : ((rows <= 32 || fp8) ? 2 : 4); }
 
 template <typename QT, typename KVT>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  switch (row_blocks_for(p.rows)) {
+  switch (row_blocks_for(p.rows, Geom<KVT>::FP8)) {
     case 1: return launch_t3<QT, KVT, 1>(p, ws_prefix, skip_combine, s);
     case 2: return launch_t3<QT, KVT, 2>(p, ws_prefix, skip_combine, s);
     default: return launch_t3<QT, KVT, 4>(p, ws_prefix, skip_combine, s);
@@ -810,11 +810,11 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 // Number of equal ranges the tile stream is cut into: one wave per (range, kv head, row group), sized so
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
 int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
-  const int nrb = row_blocks_for(rows);
+  const int nrb = row_blocks_for(rows, kv_dtype == MI355_DT_FP8_E4M3FN);
   const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
   // resident waves per CU: eight for the fp8 single-row-block kernel (LDS-limited, ~160 VGPRs), otherwise four
   // (LDS-limited with a 16-bit cache, register-limited -- one wave per SIMD -- with more than one row block)
-  const int waves_per_cu = (kv_dtype == MI355_DT_FP8_E4M3FN && nrb == 1) ? 8 : 4;
+  const int waves_per_cu = (kv_dtype == MI355_DT_FP8_E4M3FN && nrb <= 2) ? 8 : 4;
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
