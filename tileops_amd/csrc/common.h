@@ -33,6 +33,7 @@ struct DecodeParams {
   float softcap;      // 0 = off
   float cap_log2e;    // softcap * log2e
   float inv_cap_scale;  // sm_scale / softcap
+  int negate_q;         // MFMA kernel: flip the sign of the query (set by its launcher for a negative scale)
   int causal;
   // generic kernel: fixed-length KV splits per sequence
   int max_splits;

@@ -62,8 +62,8 @@ template <> struct Mma<bf16_tag> {
   static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {  // one v_cvt_pk_bf16_f32 (round to nearest even)
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
   }
   static __device__ __forceinline__ uint32_t from_fp8(uint32_t w, bool hi) {
     bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
@@ -74,8 +74,8 @@ template <> struct Mma<fp16_tag> {
   static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return (uint32_t)f32_to_fp16_bits(lo) | ((uint32_t)f32_to_fp16_bits(hi) << 16);
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {  // one v_cvt_pk_f16_f32 (round to nearest even)
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
   }
   static __device__ __forceinline__ uint32_t from_fp8(uint32_t w, bool hi) {
     f16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
@@ -125,11 +125,23 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // second, v_permlane32_swap exchanges the upper half of the first with the lower half of the second.  Fed the
 // same value twice they return (x of the even partner, x of the odd partner), so one max/add finishes a step
 // without touching the LDS crossbar.
+// Maxima as single instructions.  fmaxf() first quiets a possible signalling NaN in each operand whose origin
+// the compiler cannot see (one extra v_max per operand); the scores here are MFMA results or -inf.
+__device__ __forceinline__ float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float group_max(float x) {
   u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  x = max2(__uint_as_float(r[0]), __uint_as_float(r[1]));
   r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  return max2(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float group_sum(float x) {
   u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -148,9 +160,18 @@ __device__ __forceinline__ int part_of(int64_t u, int64_t T, int64_t NP) { retur
 __device__ __forceinline__ int part_begin(int64_t p, int64_t T, int64_t NP) { return (int)(p * T / NP); }
 
 // Position in the tile stream: sequence b, tile j of nt, plus the logical page / in-page offset of tile j.
+// lens holds seqlens[lens_base + lane]: moving to the next sequence is a register read (v_readlane), not a global
+// load whose wait would also drain every direct-to-LDS load in flight.
 struct Cursor {
   int b, j, nt, len, pg, off;
+  int lens_base, lens;
 };
+
+__device__ __forceinline__ void cursor_load_lens(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int base) {
+  const int lane = threadIdx.x & 63;
+  c.lens_base = base;
+  c.lens = seqlens[min(base + lane, batch - 1)];
+}
 
 __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int page_size, bool ps16) {
   c.j++;
@@ -176,7 +197,8 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict
       c.len = 0;
       return;
     }
-    c.len = uni(seqlens[c.b]);
+    if (c.b - c.lens_base >= 64) cursor_load_lens(c, seqlens, batch, c.b);  // once per 64 sequences
+    c.len = __builtin_amdgcn_readlane(c.lens, c.b - c.lens_base);
     c.nt = units_of(c.len);
   } while (c.nt == 0);
 }
@@ -193,6 +215,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   const int wave = uni(threadIdx.x >> 6);
   // Workgroups are dealt round-robin to the 8 XCDs, so neighbouring partitions (which read neighbouring pages of
   // a sequence) spread over all L2s and memory channels; renumbering them XCD-contiguously measured slower.
+#ifdef MI355_PHASE_TIMERS
+  const uint64_t tm_kernel0 = __builtin_readcyclecounter();
+#endif
   const int gw = blockIdx.x * NW + wave;
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int per_part = p.heads_kv * n_rg;
@@ -269,7 +294,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     b0 = uni(b0);
     pre0 = uni(pre0);
     start.b = b0;
-    start.len = uni(p.seqlens[b0]);
+    cursor_load_lens(start, p.seqlens, p.batch, b0);
+    start.len = __builtin_amdgcn_readlane(start.lens, 0);
     start.nt = units_of(start.len);
     start.j = u0 - pre0;
     if (ps16) {
@@ -401,6 +427,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   int limit[NRB];
   const int qoff = (p.causal && p.q_len > 1) ? p.q_len - 1 : 0;
   const bool softcap = p.softcap > 0.f;
+  const uint32_t q_sign = p.negate_q ? 0x80008000u : 0u;
 
   auto begin_segment = [&](const Cursor& cu) __attribute__((always_inline)) {
 #pragma unroll
@@ -428,15 +455,27 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) asm volatile("" : "+v"(qreg[rb][j]));
+      for (int j = 0; j < 4; j++) {
+        asm volatile("" : "+v"(qreg[rb][j]));
+        // a negative softmax scale is carried by the query (an exact sign flip), so the scale itself is positive
+        qreg[rb][j] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
+      }
   };
 
   // SOFF = byte offset of the stage slot inside the wave's LDS ring; a literal at every call site of the
   // single-row-block kernels (folds into the ds_read immediates), a run-time value in the multi-row-block ones
-  auto compute = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) {
+  // The stage body is split in two.  score_step: LDS reads, S^T = K.Q^T, online softmax; leaves V^T operands and
+  // packed probabilities in registers and returns whether any row moved its softmax reference (wave-uniform).
+  // value_step: O^T += V^T.P^T.  Between them the caller rescales the accumulators when asked to -- outside the
+  // steady-state loop, because the accumulators live in accumulation registers that the vector ALU cannot
+  // address, and a rescale inside the loop makes the register allocator shuttle all of them on every iteration.
+  u32x4 va_op[8];
+  u32x4 pk[NRB];
+  float alpha[NRB];
+  auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
-    u32x4 ka_op[2][4], va_op[8];
+    u32x4 ka_op[2][4];
     f32x4 ksc[2], vsc[2];
     if (!FP8) {
 #pragma unroll
@@ -504,8 +543,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
         }
     // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
     const bool need_mask = tok0 + kCT > cu.len - qoff;
-    u32x4 pk[NRB];
-    float alpha[NRB];
+    const float exp_scale = softcap ? 1.0f : p.score_scale;
+    bool any_moved = false;
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       float x[2][4];
@@ -517,16 +556,14 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
           if (FP8) s *= ksc[tb][i];
           x[tb][i] = s;
         }
+      // Without softcap the scores stay unscaled here: the (positive) scale sm_scale*log2e commutes with the
+      // maximum and is applied inside the exponent as one fused multiply-add per element.
       if (softcap) {
+        asm volatile("");  // keeps this a real (wave-uniform) branch: the tanh is too long to compute speculatively
 #pragma unroll
         for (int tb = 0; tb < 2; tb++)
 #pragma unroll
           for (int i = 0; i < 4; i++) x[tb][i] = to_logit2<true>(x[tb][i], p.score_scale, p.cap_log2e, p.inv_cap_scale);
-      } else {
-#pragma unroll
-        for (int tb = 0; tb < 2; tb++)
-#pragma unroll
-          for (int i = 0; i < 4; i++) x[tb][i] *= p.score_scale;
       }
       if (need_mask) {  // only the last tile(s) of a sequence
 #pragma unroll
@@ -541,8 +578,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       l_run[rb] += x[0][1];
       continue;
 #endif
-      float mt = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])), fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
-      mt = group_max(mt);
+      float mt = max2(max3(x[0][0], x[0][1], x[0][2]), max3(x[0][3], x[1][0], max3(x[1][1], x[1][2], x[1][3])));
+      mt = group_max(mt) * exp_scale;
       // Lazy rescale: the running reference m_run only moves when the tile maximum exceeds it by more than
       // kRescaleGap (log2 domain).  Probabilities are then at most 2^kRescaleGap instead of 1 -- harmless for
       // fp32 accumulators and 16-bit P -- and because l_run uses the same reference the final O/l is unchanged.
@@ -551,12 +588,13 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       const float m_new = moved ? mt : m_run[rb];
       alpha[rb] = moved ? fast_exp2(m_run[rb] - m_new) : 1.0f;
       m_run[rb] = m_new;
+      any_moved |= moved;
       float psum = 0.f;
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          float pr = fast_exp2(x[tb][i] - m_new);
+          float pr = fast_exp2(__builtin_fmaf(x[tb][i], exp_scale, -m_new));
           psum += pr;
           x[tb][i] = FP8 ? pr * vsc[tb][i] : pr;
         }
@@ -565,19 +603,19 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       pk[rb][1] = Mma<QT>::pack(x[0][2], x[0][3]);
       pk[rb][2] = Mma<QT>::pack(x[1][0], x[1][1]);
       pk[rb][3] = Mma<QT>::pack(x[1][2], x[1][3]);
-      if (__builtin_expect(__any(moved), 0)) {  // wave-uniform: some row of this row block moved its reference
-        // The accumulators live in accumulation registers, which the vector ALU cannot address: the two empty
-        // asm statements pin them there on entry and exit, so the copies out and back stay inside this rarely
-        // taken block instead of being hoisted into every loop iteration.
-#pragma unroll
-        for (int db = 0; db < 8; db++) {
-          asm volatile("" : "+a"(o_acc[rb][db]));
-          o_acc[rb][db] *= alpha[rb];
-          asm volatile("" : "+a"(o_acc[rb][db]));
-        }
-      }
     }
-    // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------
+    return __any(any_moved);
+  };
+  auto rescale = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+      for (int db = 0; db < 8; db++) {
+        o_acc[rb][db] *= alpha[rb];  // alpha is 1 for rows that kept their reference
+        __builtin_amdgcn_sched_barrier(0);  // one tile at a time: keeps the copies out of the accumulation registers short-lived
+      }
+  };
+  auto value_step = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int db = 0; db < 8; db++)
 #pragma unroll
@@ -642,38 +680,82 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     else if (ahead == 1) wait_vmcnt<G::IPS>();
     else wait_vmcnt<0>();
   };
-  auto run_compute = [&](int ring) __attribute__((always_inline)) {
+  auto run_score_step = [&](int ring) __attribute__((always_inline)) -> bool {
 #ifndef MI355_DEBUG_NO_COMPUTE
     if constexpr (NRB == 1) {
-      // one copy of the stage body per ring slot: the slot offset folds into the LDS read immediates
-      if (ring == 0) compute(0u, cc);
-      else if (NS > 1 && ring == 1) compute((uint32_t)G::STAGE, cc);
-      else if (NS > 2 && ring == 2) compute(2u * G::STAGE, cc);
-      else compute(3u * G::STAGE, cc);
+      // one copy of the body per ring slot: the slot offset folds into the LDS read immediates
+      if (ring == 0) return score_step(0u, cc);
+      else if (NS > 1 && ring == 1) return score_step((uint32_t)G::STAGE, cc);
+      else if (NS > 2 && ring == 2) return score_step(2u * G::STAGE, cc);
+      else return score_step(3u * G::STAGE, cc);
     } else {
-      compute((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
+      return score_step((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
     }
+#else
+    return false;
 #endif
   };
+  auto run_value_step = [&]() __attribute__((always_inline)) {
+#ifndef MI355_DEBUG_NO_COMPUTE
+    value_step();
+#endif
+  };
+#ifdef MI355_PHASE_TIMERS
+  // measurement build only: per-wave cycle totals of the loop phases, left behind the workspace proper
+  uint64_t tm_issue = 0, tm_wait = 0, tm_comp = 0, tm_seg = 0, tm_mark = __builtin_readcyclecounter();
+  const uint64_t tm_loop0 = tm_mark;
+#define TM(acc) { uint64_t now_ = __builtin_readcyclecounter(); acc += now_ - tm_mark; tm_mark = now_; }
+#else
+#define TM(acc)
+#endif
   int u = 0, ring = 0, seg_count = 0;
   while (u < n_units) {
     const int seg_first_j = cc.j;
     const int seg_units = min(cc.nt - cc.j, n_units - u);
     issue_ahead(ring);   // before the query loads, so the next tile is already in flight while they land
+    TM(tm_issue)
     begin_segment(cc);
-    for (int k = 0; k < seg_units; ++k) {
-      if (k > 0) issue_ahead(ring);
-      wait_stage(u);
-      run_compute(ring);
-      ++u;
-      ++cc.j;
-      ring = ring + 1 == NS ? 0 : ring + 1;
+    TM(tm_seg)
+    int k = 0;
+    while (k < seg_units) {
+      bool moved = false;
+      for (; k < seg_units; ++k) {  // steady state: no tile in here rescales the accumulators
+        if (k > 0) issue_ahead(ring);
+        TM(tm_issue)
+        wait_stage(u);
+        TM(tm_wait)
+        moved = run_score_step(ring);
+        if (__builtin_expect(moved, 0)) break;
+        run_value_step();
+        TM(tm_comp)
+        ++u;
+        ++cc.j;
+        ring = ring + 1 == NS ? 0 : ring + 1;
+      }
+      if (moved) {  // rare after the first tiles of a sequence: finish this tile out of line, then re-enter
+        rescale();
+        run_value_step();
+        TM(tm_comp)
+        ++u;
+        ++cc.j;
+        ring = ring + 1 == NS ? 0 : ring + 1;
+        ++k;
+      }
     }
     --cc.j;  // end_segment and cursor_next see the last tile of the segment
     end_segment(cc, seg_first_j == 0 && cc.j == cc.nt - 1, seg_count == 0 ? 0 : 1);
     ++seg_count;
     cursor_next(cc, p.seqlens, p.batch, p.page_size, ps16);
+    TM(tm_seg)
   }
+#ifdef MI355_PHASE_TIMERS
+  if (lane == 0) {
+    float* dst = (float*)(ws_prefix + ((p.batch + 1) * 4 + 63) / 64 * 64) + (size_t)gw * 8;  // past the records: caller over-allocates
+    dst[0] = (float)tm_issue; dst[1] = (float)tm_wait; dst[2] = (float)tm_comp; dst[3] = (float)tm_seg;
+    dst[4] = (float)(tm_loop0 - tm_kernel0); dst[5] = (float)(tm_mark - tm_kernel0); dst[6] = (float)n_units; dst[7] = (float)seg_count;
+  }
+#endif
+#undef TM
 }
 
 // Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
@@ -828,6 +910,12 @@ size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int ba
 
 const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, bool skip_combine, hipStream_t s) {
   DecodeParams p = p_in;
+  // The kernel applies the score scale after taking row maxima, which needs it positive: move the sign into the
+  // query, and replace a zero scale (uniform attention) by a tiny positive one so masked -inf scores stay -inf.
+  float& signed_scale = p.softcap > 0.f ? p.inv_cap_scale : p.score_scale;
+  p.negate_q = signed_scale < 0.f ? 1 : 0;
+  signed_scale = fabsf(signed_scale);
+  if (!(p.softcap > 0.f) && signed_scale < 1e-30f) signed_scale = 1e-30f;
   size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
   char* ws = (char*)p_in.part_o;
   p.part_o = (float*)ws;
