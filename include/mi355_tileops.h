@@ -104,6 +104,32 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
                            int kernel, void* hip_stream);
 
 /*
+ * GQA decode over a contiguous (un-paged) KV cache: one call = one forward of
+ * GroupedQueryAttentionDecodeWithKVCacheFwdOp (src/tileops/ops/attention/gqa.py:1336-1350 ->
+ * GQADecodeKernel.forward, src/tileops/kernels/attention/gqa_decode.py:555-612; custom-op argument lists
+ * :312-335, :358-385), i.e. the reference's no-split kernel (:24-122), split kernel (:124-310) and its combine.
+ * Same kernels as the paged entry point with identity addressing: sequence b occupies tokens
+ * [b*kv_seq_stride, b*kv_seq_stride + real_seqlen_kv) of k and v.
+ *
+ *   q              [batch, q_len, heads, dim]  q_dtype, contiguous (q_len == 1 is the reference op)
+ *   k, v           [batch, kv_seq_stride, heads_kv, dim]  kv_dtype, contiguous; only the first real_seqlen_kv tokens
+ *                  of each sequence are read, so no zero padding up to a compiled-in length is needed
+ *                  (the reference pads to seqlen_kv, gqa.py:1338-1345)
+ *   k_scale,
+ *   v_scale        [batch, kv_seq_stride, heads_kv] fp32, iff kv_dtype == MI355_DT_FP8_E4M3FN (this library's extension)
+ *   real_seqlen_kv tokens of context of every sequence (one value, as in the reference's forward)
+ *   workspace      >= what mi355_gqa_decode_workspace() reports for max_seqlen_kv >= real_seqlen_kv
+ * The remaining arguments are those of mi355_gqa_paged_decode().
+ */
+int mi355_gqa_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int64_t max_seqlen_kv, int q_dtype,
+                               int kv_dtype, int num_split_in, int kernel, size_t* workspace_bytes, int* num_split_out,
+                               int* kernel_out);
+int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale, void* out,
+                     void* workspace, size_t workspace_bytes, int batch, int q_len, int heads, int heads_kv, int dim,
+                     int64_t kv_seq_stride, int real_seqlen_kv, int q_dtype, int kv_dtype, float sm_scale, float softcap,
+                     int causal, int num_split, int kernel, void* hip_stream);
+
+/*
  * Index-probe: materialise the logical KV rows a decode call would read, with the same device page
  * arithmetic the attention kernels use.  dense_out [batch, max_len, heads_kv * dim] elem_bytes-wide
  * elements; rows t >= seqlens[b] are left untouched.  Lets a test compare the gather bit-for-bit with

@@ -1,6 +1,6 @@
 """MI355X (gfx950) paged GQA decode attention behind the TileOPs operator contract.
 
-Public surface: the two ops, the backend seam, the manifest loader.  The HIP library is opened lazily on
+Public surface: the three ops, the backend seam, the manifest loader.  The HIP library is opened lazily on
 the first kernel build; importing this package touches no device.
 """
 
@@ -9,11 +9,13 @@ from .backend import (  # noqa: F401
     default_target, load_failures, register_detector, register_kernel_builder, registered_targets, set_default_target,
 )
 from .ops import (  # noqa: F401
+    GroupedQueryAttentionDecodeWithKVCacheFwdOp,
     GroupedQueryAttentionDecodePagedWithKVCacheFwdOp,
     GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp,
 )
 
 __all__ = [
+    "GroupedQueryAttentionDecodeWithKVCacheFwdOp",
     "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp",
     "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp",
 ]

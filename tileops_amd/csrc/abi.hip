@@ -89,55 +89,23 @@ int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_s
   return MI355_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int mi355_abi_version(void) { return MI355_ABI_VERSION; }
-
-const char* mi355_last_error(void) { return g_err; }
-
-int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
-                                     int64_t max_blocks_per_seq, int q_dtype, int kv_dtype, int num_split_in, int kernel,
-                                     size_t* workspace_bytes, int* num_split_out, int* kernel_out) {
-  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
-  if (rc) return rc;
-  Plan plan;
-  // softcap does not change the plan; the MFMA kernel serves both settings
-  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in,
-                 kernel & ~MI355_KERNEL_FLAG_SKIP_COMBINE, &plan);
-  if (rc) return rc;
-  if (workspace_bytes) *workspace_bytes = plan.part_o_bytes + plan.part_lse_bytes;
-  if (num_split_out) *num_split_out = plan.kernel == MI355_KERNEL_GENERIC ? plan.max_splits : plan.n_parts;
-  if (kernel_out) *kernel_out = plan.kernel;
-  return MI355_OK;
-}
-
-int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
-                           const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out, void* workspace,
-                           size_t workspace_bytes, int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
-                           int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale, float softcap, int causal,
-                           int num_split, int kernel, void* hip_stream) {
-  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
-  if (rc) return rc;
+// One decode call, paged (block_table/seqlens given) or contiguous (contig_stride > 0, uniform_len).
+int run_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+               const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, int64_t contig_stride,
+               int uniform_len, void* out, void* workspace, size_t workspace_bytes, int batch, int q_len, int heads,
+               int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale,
+               float softcap, int causal, int num_split, int kernel, void* hip_stream) {
   const bool skip_combine = (kernel & MI355_KERNEL_FLAG_SKIP_COMBINE) != 0;
   kernel &= ~MI355_KERNEL_FLAG_SKIP_COMBINE;
-  if (batch == 0) return MI355_OK;
-  if (!q || !k || !v || !seqlens || !block_table || !out)
-    return fail(MI355_EINVAL, "q, k, v, seqlens, block_table and out must be non-null");
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
   if (fp8 && (!k_scale || !v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale are required with an fp8 KV cache");
   if (!fp8 && (k_scale || v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale must be null unless kv_dtype is fp8_e4m3fn");
-  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
-    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens,
-                page_size);
-  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
   if (!(softcap >= 0.f)) return fail(MI355_EINVAL, "softcap must be non-negative");
   if (!(sm_scale == sm_scale)) return fail(MI355_EINVAL, "sm_scale is NaN");
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(MI355_EINVAL, "q, k, v and out must be 16-byte aligned");
   Plan plan;
-  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan);
+  int rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan);
   if (rc) return rc;
   const size_t need = plan.part_o_bytes + plan.part_lse_bytes;
   if (need > 0) {
@@ -156,6 +124,8 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
   p.seqlens = seqlens;
   p.block_table = block_table;
   p.bt_row_stride = bt_row_stride;
+  p.contig_stride = contig_stride;
+  p.uniform_len = uniform_len;
   p.out = out;
   p.part_o = (float*)workspace;
   p.part_lse = (float*)((char*)workspace + plan.part_o_bytes);
@@ -191,6 +161,80 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
   }
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
   return MI355_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_abi_version(void) { return MI355_ABI_VERSION; }
+
+const char* mi355_last_error(void) { return g_err; }
+
+int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                                     int64_t max_blocks_per_seq, int q_dtype, int kv_dtype, int num_split_in, int kernel,
+                                     size_t* workspace_bytes, int* num_split_out, int* kernel_out) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
+  if (rc) return rc;
+  Plan plan;
+  // softcap does not change the plan; the MFMA kernel serves both settings
+  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in,
+                 kernel & ~MI355_KERNEL_FLAG_SKIP_COMBINE, &plan);
+  if (rc) return rc;
+  if (workspace_bytes) *workspace_bytes = plan.part_o_bytes + plan.part_lse_bytes;
+  if (num_split_out) *num_split_out = plan.kernel == MI355_KERNEL_GENERIC ? plan.max_splits : plan.n_parts;
+  if (kernel_out) *kernel_out = plan.kernel;
+  return MI355_OK;
+}
+
+int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                           const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out, void* workspace,
+                           size_t workspace_bytes, int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                           int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale, float softcap, int causal,
+                           int num_split, int kernel, void* hip_stream) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
+  if (rc) return rc;
+  if (batch == 0) return MI355_OK;
+  if (!q || !k || !v || !seqlens || !block_table || !out)
+    return fail(MI355_EINVAL, "q, k, v, seqlens, block_table and out must be non-null");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens,
+                page_size);
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  return run_decode(q, k, v, k_scale, v_scale, seqlens, block_table, bt_row_stride, 0, 0, out, workspace, workspace_bytes,
+                    batch, q_len, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype, kv_dtype, sm_scale, softcap,
+                    causal, num_split, kernel, hip_stream);
+}
+
+// A contiguous cache is walked in 32-token tiles: the "page size" both kernels do their tile arithmetic with.
+static const int kContigTile = 32;
+
+int mi355_gqa_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int64_t max_seqlen_kv, int q_dtype,
+                               int kv_dtype, int num_split_in, int kernel, size_t* workspace_bytes, int* num_split_out,
+                               int* kernel_out) {
+  if (max_seqlen_kv <= 0) return fail(MI355_EINVAL, "max_seqlen_kv must be positive");
+  return mi355_gqa_paged_decode_workspace(batch, q_len, heads, heads_kv, dim, kContigTile,
+                                          (max_seqlen_kv + kContigTile - 1) / kContigTile, q_dtype, kv_dtype, num_split_in,
+                                          kernel, workspace_bytes, num_split_out, kernel_out);
+}
+
+int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale, void* out,
+                     void* workspace, size_t workspace_bytes, int batch, int q_len, int heads, int heads_kv, int dim,
+                     int64_t kv_seq_stride, int real_seqlen_kv, int q_dtype, int kv_dtype, float sm_scale, float softcap,
+                     int causal, int num_split, int kernel, void* hip_stream) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, kContigTile, q_dtype, kv_dtype);
+  if (rc) return rc;
+  if (batch == 0) return MI355_OK;
+  if (!q || !k || !v || !out) return fail(MI355_EINVAL, "q, k, v and out must be non-null");
+  if (real_seqlen_kv < 0) return fail(MI355_EINVAL, "real_seqlen_kv must be non-negative, got %d", real_seqlen_kv);
+  if (kv_seq_stride <= 0 || kv_seq_stride < real_seqlen_kv)
+    return fail(MI355_EINVAL, "kv_seq_stride (%lld) must be positive and at least real_seqlen_kv (%d)",
+                (long long)kv_seq_stride, real_seqlen_kv);
+  const int64_t max_blocks = ((int64_t)real_seqlen_kv + kContigTile - 1) / kContigTile;
+  return run_decode(q, k, v, k_scale, v_scale, nullptr, nullptr, max_blocks > 0 ? max_blocks : 1, kv_seq_stride,
+                    real_seqlen_kv, out, workspace, workspace_bytes, batch, q_len, heads, heads_kv, dim, kContigTile,
+                    (int64_t)batch * kv_seq_stride, q_dtype, kv_dtype, sm_scale, softcap, causal, num_split, kernel,
+                    hip_stream);
 }
 
 int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,

@@ -22,6 +22,10 @@ struct DecodeParams {
   const int32_t* seqlens;
   const int32_t* block_table;
   int64_t bt_row_stride;
+  // Contiguous cache (no block table): block_table and seqlens are null, sequence b occupies tokens
+  // [b*contig_stride, b*contig_stride + uniform_len) of k/v, and page_size is only the tile granule.
+  int64_t contig_stride;
+  int uniform_len;
   void* out;
   float* part_o;    // workspace: normalised partial outputs, fp32
   float* part_lse;  // workspace: log2-domain log-sum-exp per partial (-inf = empty)
@@ -41,6 +45,9 @@ struct DecodeParams {
   // MFMA kernel: even partition of the KV tile stream
   int n_parts;
 };
+
+// Context length of sequence b: per-sequence array (paged cache) or one value for all (contiguous cache).
+__device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) { return p.seqlens ? p.seqlens[b] : p.uniform_len; }
 
 // Number of KV splits of one sequence and the (tile-aligned) tokens per split, generic kernel.
 // Used identically by the attention kernel and its combine kernel.

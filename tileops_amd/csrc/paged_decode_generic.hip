@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
   const int n_rowblk = (p.rows + RB - 1) / RB;
   const int kvh = blockIdx.x / n_rowblk, r0 = (blockIdx.x % n_rowblk) * RB;
   const int split = blockIdx.y, b = blockIdx.z;
-  const int len = p.seqlens[b];
+  const int len = seq_len_of(p, b);
   int n_splits, chunk;
   split_geometry(len, p.split_tokens, p.max_splits, &n_splits, &chunk);
   if (split >= n_splits) return;
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
   }
 
   for (int t = t_begin + gi; t < t_end; t += 16) {
-    const int64_t phys = physical_token(bt_row, t, p.page_size, p.n_pages);
+    const int64_t phys = p.contig_stride ? (int64_t)b * p.contig_stride + t : physical_token(bt_row, t, p.page_size, p.n_pages);
     const int64_t row = phys * p.heads_kv + kvh;
     uint32_t kraw[EPL * KB / 4], vraw[EPL * KB / 4];
     load_raw<EPL * KB>((const char*)p.k + (row * D + c * EPL) * KB, kraw);
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
 template <typename QT>
 __global__ void paged_decode_generic_combine_kernel(const DecodeParams p) {
   const int b = blockIdx.y, grow_in = blockIdx.x, d = threadIdx.x;
-  const int len = p.seqlens[b];
+  const int len = seq_len_of(p, b);
   int n_splits, chunk;
   split_geometry(len, p.split_tokens, p.max_splits, &n_splits, &chunk);
   if (n_splits == 1) return;  // the attention kernel wrote the output directly

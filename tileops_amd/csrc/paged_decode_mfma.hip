@@ -167,13 +167,14 @@ struct Cursor {
   int lens_base, lens;
 };
 
-__device__ __forceinline__ void cursor_load_lens(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int base) {
+__device__ __forceinline__ void cursor_load_lens(Cursor& c, const DecodeParams& p, int base) {
   const int lane = threadIdx.x & 63;
   c.lens_base = base;
-  c.lens = seqlens[min(base + lane, batch - 1)];
+  c.lens = seq_len_of(p, min(base + lane, p.batch - 1));
 }
 
-__device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict__ seqlens, int batch, int page_size, bool ps16) {
+__device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bool ps16) {
+  const int batch = p.batch, page_size = p.page_size;
   c.j++;
   if (c.j < c.nt) {
     if (ps16) {
@@ -197,7 +198,7 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const int32_t* __restrict
       c.len = 0;
       return;
     }
-    if (c.b - c.lens_base >= 64) cursor_load_lens(c, seqlens, batch, c.b);  // once per 64 sequences
+    if (c.b - c.lens_base >= 64) cursor_load_lens(c, p, c.b);  // once per 64 sequences
     c.len = __builtin_amdgcn_readlane(c.lens, c.b - c.lens_base);
     c.nt = units_of(c.len);
   } while (c.nt == 0);
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   int T = 0;
   for (int base = 0; base < p.batch; base += 64) {
     int b = base + lane;
-    int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+    int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
 #pragma unroll
     for (int m = 1; m < 64; m <<= 1) n += __shfl_xor(n, m, 64);
     T += n;
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     int carry = 0;
     for (int base = 0; base < p.batch; base += 64) {
       int b = base + lane;
-      int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+      int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
       int incl = n;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     int carry = 0, b0 = -1, pre0 = 0;
     for (int base = 0; base < p.batch && b0 < 0; base += 64) {
       int b = base + lane;
-      int n = b < p.batch ? units_of(p.seqlens[b]) : 0;
+      int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
       int incl = n;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     b0 = uni(b0);
     pre0 = uni(pre0);
     start.b = b0;
-    cursor_load_lens(start, p.seqlens, p.batch, b0);
+    cursor_load_lens(start, p, b0);
     start.len = __builtin_amdgcn_readlane(start.lens, 0);
     start.nt = units_of(start.len);
     start.j = u0 - pre0;
@@ -380,6 +381,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       int last_pg = (cu.len - 1) >> 4;
       ptok0 = phys_page(cu, cu.pg) * 16;
       ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
+    } else if (p.contig_stride) {
+      ptok0 = (int64_t)cu.b * p.contig_stride + tok0;  // contiguous cache: no table, a tile never straddles anything
     } else {
       ptok0 = phys_page(cu, cu.pg) * p.page_size + cu.off;
     }
@@ -664,12 +667,12 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   int issued = 0;
   for (; issued < NS - 1 && issued < n_units; ++issued) {
     issue(ci, issued);
-    cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
+    cursor_next(ci, p, ps16);
   }
   auto issue_ahead = [&](int ring) __attribute__((always_inline)) {
     if (issued < n_units) {
       issue(ci, ring == 0 ? NS - 1 : ring - 1);  // the ring slot consumed in the previous iteration
-      cursor_next(ci, p.seqlens, p.batch, p.page_size, ps16);
+      cursor_next(ci, p, ps16);
       ++issued;
     }
   };
@@ -745,7 +748,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     --cc.j;  // end_segment and cursor_next see the last tile of the segment
     end_segment(cc, seg_first_j == 0 && cc.j == cc.nt - 1, seg_count == 0 ? 0 : 1);
     ++seg_count;
-    cursor_next(cc, p.seqlens, p.batch, p.page_size, ps16);
+    cursor_next(cc, p, ps16);
     TM(tm_seg)
   }
 #ifdef MI355_PHASE_TIMERS

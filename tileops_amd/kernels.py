@@ -24,12 +24,15 @@ import torch
 from . import native
 
 __all__ = [
-    "AttentionCall", "GQADecodePagedKernel", "GQADecodePagedMfmaKernel", "Kernel", "PAGED_DECODE_KEYS",
+    "AttentionCall", "DECODE_KEYS", "GQADecodeKernel", "GQADecodeMfmaKernel", "GQADecodePagedKernel",
+    "GQADecodePagedMfmaKernel", "Kernel", "PAGED_DECODE_KEYS",
     "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch",
 ]
 
 #: Dispatch keys of the paged decode ops, in no particular order (selection never reads the order).
 PAGED_DECODE_KEYS = ("gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel")
+#: Dispatch keys of the contiguous-cache decode op.
+DECODE_KEYS = ("gqa_decode_kernel", "gqa_decode_mfma_kernel")
 
 GFX950_ARCH = 95  # torch.cuda.get_device_capability() == (9, 5) on gfx950
 
@@ -51,7 +54,7 @@ def _as_torch_dtype(dtype: Any) -> torch.dtype:
 
 @dataclass(frozen=True)
 class AttentionCall:
-    """Facts of one paged decode call that kernel selection filters on
+    """Facts of one decode call that kernel selection filters on (``page_size`` 0 = contiguous cache)
     (reference: src/tileops/kernels/attention/call_spec.py:44-76, kernels/call_spec.py:8-42)."""
 
     dtype: torch.dtype
@@ -290,6 +293,131 @@ class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
     @property
     def default_config(self) -> dict[str, Any]:
         return {"block_N": gqa_decode_paged_block_n(self.page_size), "num_split": 0}
+
+    @property
+    def autotune_configs(self) -> list[dict]:
+        return [dict(self.default_config)]
+
+
+class GQADecodeKernel(Kernel):
+    """General GQA decode over a contiguous ``[batch, N_kv, heads_kv, dim]`` cache on gfx950: the VALU HIP kernel
+    with identity addressing plus the fp32 split-KV combine.
+
+    Constructor arguments and the default split policy follow the reference class
+    (src/tileops/kernels/attention/gqa_decode.py:426-449, :511-553); ``groups`` is the number of KV heads, as
+    there.  ``forward(Q, K, V, real_seqlen_kv)`` reads only the first ``real_seqlen_kv`` tokens of each
+    sequence, so the cache needs no padding up to ``seqlen_kv``.  ``kv_dtype`` is this package's FP8 extension.
+    """
+
+    supported_archs = [GFX950_ARCH]
+    general = True
+    _native_kernel = native.KERNEL_GENERIC
+
+    def __init__(self, batch: int, heads: int, groups: int, seqlen_kv: int, dim: int, dtype: Any = "float16",
+                 sm_scale: Optional[float] = None, softcap: float = 0.0, config: Optional[dict] = None,
+                 tune: bool = False, *, kv_dtype: Any = None, device_index: Optional[int] = None) -> None:
+        super().__init__(device_index=device_index)
+        self.batch, self.heads, self.groups, self.seqlen_kv, self.dim = batch, heads, groups, seqlen_kv, dim
+        self.dtype = _as_torch_dtype(dtype)
+        self.kv_dtype = self.dtype if kv_dtype is None else _as_torch_dtype(kv_dtype)
+        self.sm_scale = dim ** -0.5 if sm_scale is None else sm_scale
+        self.softcap = softcap
+        if self.groups <= 0:
+            raise ValueError("groups must be positive")
+        if self.heads % self.groups != 0:
+            raise ValueError("heads must be divisible by groups")
+        if self.seqlen_kv <= 0:
+            raise ValueError("seqlen_kv must be positive")
+        self._plans: dict[int, tuple[int, int]] = {}
+        self.init_config(config, tune)
+
+    def _default_num_split(self) -> int:
+        """Reference policy (gqa_decode.py:520-532): 32 splits for single-request decode with at most two KV
+        heads and a query group of at least eight, 16 otherwise, never more than there are tokens."""
+        kv_group_num = self.heads // self.groups
+        candidate = 32 if (self.batch == 1 and self.dim == 128 and self.groups <= 2 and kv_group_num >= 8) else 16
+        return min(candidate, self.seqlen_kv)
+
+    @property
+    def default_config(self) -> dict[str, Any]:
+        return {"num_split": self._default_num_split()}
+
+    @property
+    def autotune_configs(self) -> list[dict]:
+        return [{"num_split": ns} for ns in ([n for n in (2, 4, 8, 16, 32) if n <= self.seqlen_kv] or [1])]
+
+    def autotune(self) -> None:
+        device = torch.device("cuda", self.device_index if self.device_index is not None else torch.cuda.current_device())
+        q = torch.randn(self.batch, self.heads, self.dim, device=device, dtype=self.dtype)
+        kv = torch.randn(2, self.batch, self.seqlen_kv, self.groups, self.dim, device=device, dtype=torch.float32)
+        if self.kv_dtype == torch.float8_e4m3fn:
+            k, v = kv[0].clamp(-448, 448).to(self.kv_dtype), kv[1].clamp(-448, 448).to(self.kv_dtype)
+            ks = torch.full((self.batch, self.seqlen_kv, self.groups), 0.01, device=device, dtype=torch.float32)
+            vs = ks.clone()
+        else:
+            k, v, ks, vs = kv[0].to(self.kv_dtype), kv[1].to(self.kv_dtype), None, None
+        best, best_ms = None, float("inf")
+        for cfg in self.autotune_configs:
+            self.config = dict(cfg)
+            for _ in range(3):
+                self.forward(q, k, v, self.seqlen_kv, ks, vs)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(10):
+                self.forward(q, k, v, self.seqlen_kv, ks, vs)
+            stop.record()
+            stop.synchronize()
+            ms = start.elapsed_time(stop) / 10
+            if ms < best_ms:
+                best, best_ms = dict(cfg), ms
+        self.config = best
+
+    def _plan(self) -> tuple[int, int]:
+        key = int(self.config.get("num_split", 0))
+        plan = self._plans.get(key)
+        if plan is None:
+            nbytes, nsplit, _ = native.contiguous_decode_workspace(
+                self.batch, 1, self.heads, self.groups, self.dim, self.seqlen_kv, self.dtype, self.kv_dtype, key,
+                self._native_kernel)
+            plan = self._plans[key] = (nbytes, nsplit)
+        return plan
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: int,
+                k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        native.require_gfx950(q.device)
+        if real_seqlen_kv > self.seqlen_kv:
+            raise ValueError(f"real_seqlen_kv={real_seqlen_kv} exceeds the seqlen_kv={self.seqlen_kv} this kernel was built for")
+        nbytes, nsplit = self._plan()
+        out = torch.empty_like(q)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
+        native.contiguous_decode(
+            q, k, v, k_scale, v_scale, out, workspace, batch=self.batch, q_len=1, heads=self.heads, heads_kv=self.groups,
+            dim=self.dim, real_seqlen_kv=real_seqlen_kv, sm_scale=self.sm_scale, softcap=self.softcap, causal=True,
+            num_split=nsplit, kernel=self._native_kernel)
+        return out
+
+
+class GQADecodeMfmaKernel(GQADecodeKernel):
+    """MFMA GQA decode over a contiguous cache: the paged MFMA kernel with identity addressing.  Takes the place of
+    the reference's specialised sibling (``GQADecodeBs1Kernel``, src/tileops/kernels/attention/gqa_decode_bs1.py):
+    it states the narrower region it serves (head_dim 128, ...) and wins there, for any batch."""
+
+    general = False
+    _native_kernel = native.KERNEL_MFMA
+
+    @classmethod
+    def applies(cls, call: AttentionCall) -> bool:
+        try:
+            native.contiguous_decode_workspace(call.batch, call.q_len, call.heads, call.heads_kv, call.dim,
+                                               max(call.seqlen_kv, 1), call.dtype, call.kv_dtype or call.dtype, 0,
+                                               native.KERNEL_MFMA)
+        except (NotImplementedError, ValueError):
+            return False
+        return True
+
+    @property
+    def default_config(self) -> dict[str, Any]:
+        return {"num_split": 0}  # the tile stream is cut evenly over the chip; there is nothing to choose
 
     @property
     def autotune_configs(self) -> list[dict]:

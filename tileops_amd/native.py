@@ -27,6 +27,8 @@ EXPORTED_SYMBOLS = (
     "mi355_last_error",
     "mi355_gqa_paged_decode_workspace",
     "mi355_gqa_paged_decode",
+    "mi355_gqa_decode_workspace",
+    "mi355_gqa_decode",
     "mi355_gather_probe",
     "mi355_kv_append_fp8",
 )
@@ -56,6 +58,17 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.mi355_gqa_paged_decode.argtypes = [
         _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
+        _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
+    ]
+    lib.mi355_gqa_decode_workspace.restype = _c_int
+    lib.mi355_gqa_decode_workspace.argtypes = [
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int,
+        ctypes.POINTER(_c_sz), ctypes.POINTER(_c_int), ctypes.POINTER(_c_int),
+    ]
+    lib.mi355_gqa_decode.restype = _c_int
+    lib.mi355_gqa_decode.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_sz,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int,
         _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
     ]
     lib.mi355_gather_probe.restype = _c_int
@@ -162,6 +175,38 @@ def paged_decode(
         workspace.data_ptr() if workspace is not None else None,
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
         batch, q_len, heads, heads_kv, dim, page_size, k.shape[0],
+        dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
+        int(num_split), int(kernel), _stream_ptr(q.device)))
+
+
+def contiguous_decode_workspace(
+    batch: int, q_len: int, heads: int, heads_kv: int, dim: int, max_seqlen_kv: int,
+    q_dtype: torch.dtype, kv_dtype: torch.dtype, num_split: int = 0, kernel: int = KERNEL_AUTO,
+) -> tuple[int, int, int]:
+    """(workspace_bytes, num_split, kernel) for a contiguous-cache decode call.  Touches no device."""
+    lib = load()
+    nbytes, nsplit, kout = _c_sz(0), _c_int(0), _c_int(0)
+    _check(lib.mi355_gqa_decode_workspace(
+        batch, q_len, heads, heads_kv, dim, max_seqlen_kv, dtype_code(q_dtype), dtype_code(kv_dtype),
+        num_split, kernel, ctypes.byref(nbytes), ctypes.byref(nsplit), ctypes.byref(kout)))
+    return int(nbytes.value), int(nsplit.value), int(kout.value)
+
+
+def contiguous_decode(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
+    out: torch.Tensor, workspace: Optional[torch.Tensor], *, batch: int, q_len: int, heads: int, heads_kv: int, dim: int,
+    real_seqlen_kv: int, sm_scale: float, softcap: float, causal: bool, num_split: int, kernel: int,
+) -> None:
+    """Enqueue one contiguous-cache decode call (``k``/``v`` ``[batch, N_kv, heads_kv, dim]``) on the current stream."""
+    lib = load()
+    _check(lib.mi355_gqa_decode(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        out.data_ptr(),
+        workspace.data_ptr() if workspace is not None else None,
+        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        batch, q_len, heads, heads_kv, dim, k.shape[1], int(real_seqlen_kv),
         dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
         int(num_split), int(kernel), _stream_ptr(q.device)))
 

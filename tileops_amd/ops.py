@@ -24,10 +24,14 @@ from typing import Dict, Optional
 import torch
 
 from .backend import Target
-from .kernels import PAGED_DECODE_KEYS, AttentionCall, GQADecodePagedKernel, GQADecodePagedMfmaKernel, get_arch
+from .kernels import (
+    DECODE_KEYS, PAGED_DECODE_KEYS, AttentionCall, GQADecodeKernel, GQADecodeMfmaKernel, GQADecodePagedKernel,
+    GQADecodePagedMfmaKernel, get_arch,
+)
 from .op_base import _UNRESOLVED, Op
 
 __all__ = [
+    "GroupedQueryAttentionDecodeWithKVCacheFwdOp",
     "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp",
     "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp",
 ]
@@ -246,3 +250,113 @@ class GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp(_PagedDecodeOp)
                 block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
                 v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         return self._run(q, k, v, real_seqlen_kv, block_table, k_scale, v_scale)
+
+
+class GroupedQueryAttentionDecodeWithKVCacheFwdOp(Op):
+    """GQA decode over a contiguous KV cache.  Layout: Q ``[batch, heads, dim]``; K, V ``[batch, N_kv, heads_kv, dim]``
+    (BSHD) with ``N_kv <= seqlen_kv`` the context length of every sequence.
+
+    Keeps the reference op's contract (src/tileops/ops/attention/gqa.py:1260-1350): same constructor arguments,
+    defaults and error messages, ``forward(q, k, v)`` with the real length taken from ``k.shape[1]``, output =
+    ``q``'s shape and dtype.  The reference zero-pads K/V to the compiled ``seqlen_kv`` (:1338-1345); the kernels
+    here take the length at run time and read only the tokens that exist, so nothing is copied.  As for the paged
+    ops, K/V may be ``float8_e4m3fn`` with trailing ``k_scale, v_scale [batch, N_kv, heads_kv]`` fp32.
+    """
+
+    _seen_call: Optional[dict] = None
+
+    def __init__(self, batch: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int,
+                 sm_scale: Optional[float] = None, softcap: Optional[float] = None,
+                 kernel_map: Optional[Dict[str, type]] = None, tune: bool = False, *, target: Target = None) -> None:
+        _validate_gqa_dims(heads, heads_kv, dim)
+        self.batch, self.heads, self.heads_kv, self.seqlen_kv, self.dim = batch, heads, heads_kv, seqlen_kv, dim
+        self.sm_scale = _attention_scale(dim, sm_scale)
+        self.softcap = _score_softcap(softcap)
+        self.tune = tune
+        if target is not None:
+            self.target = target
+        self.dispatch_kernel(kernel_map)
+
+    @property
+    def default_kernel_map(self) -> Dict[str, type]:
+        return {"gqa_decode_kernel": GQADecodeKernel, "gqa_decode_mfma_kernel": GQADecodeMfmaKernel}
+
+    def attention_call(self, dtype: torch.dtype, kv_dtype: Optional[torch.dtype] = None,
+                       device: Optional[torch.device] = None) -> AttentionCall:
+        index = device.index if device is not None and device.type == "cuda" else None
+        return AttentionCall(
+            dtype=dtype, kv_dtype=kv_dtype or dtype, batch=self.batch, heads=self.heads, heads_kv=self.heads_kv,
+            seqlen_kv=self.seqlen_kv, dim=self.dim, page_size=0, sm_scale=self.sm_scale, softcap=self.softcap,
+            tune=self.tune, arch=get_arch(index))
+
+    def _get_kernel(self, inputs: "tuple[torch.Tensor | None, ...]", dtype: torch.dtype,
+                    kv_dtype: Optional[torch.dtype] = None):
+        _validate_attention_dtype(dtype)
+        kv_dtype = kv_dtype or dtype
+        if self._builder is not None and self._builder is not _UNRESOLVED:
+            return self.get_or_build_kernel("gqa_decode_kernel", inputs)
+        device = next((t.device for t in inputs if t is not None), None)
+        call = self.attention_call(dtype, kv_dtype, device)
+        key = self.select_kernel_key(DECODE_KEYS, call)
+
+        def build():
+            return self.kernel_map[key](
+                call.batch, call.heads, call.heads_kv, call.seqlen_kv, call.dim, call.dtype, sm_scale=call.sm_scale,
+                softcap=call.softcap, tune=call.tune, kv_dtype=call.kv_dtype,
+                device_index=device.index if device is not None and device.type == "cuda" else None)
+
+        return self.get_or_build_kernel(key, inputs, key=(dtype, kv_dtype), build=build)
+
+    def _infer_output_shapes(self, q_shape, k_shape, v_shape, k_scale_shape=None, v_scale_shape=None) -> dict[str, tuple[int, ...]]:
+        """Manifest ``shape_rules``: ``o.shape == q.shape``."""
+        return {"o": tuple(q_shape)}
+
+    def _validate_call(self, q, k, v, k_scale, v_scale) -> None:
+        named = {"q": q, "k": k, "v": v}
+        for name, t in named.items():
+            if not isinstance(t, torch.Tensor):
+                raise ValueError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+        self._validate_dtypes(q, k, v, k_scale, v_scale)
+        fp8 = k.dtype == FP8
+        if fp8 and (k_scale is None or v_scale is None):
+            raise ValueError("k_scale and v_scale are required when the KV cache is float8_e4m3fn")
+        if not fp8 and (k_scale is not None or v_scale is not None):
+            raise ValueError("k_scale and v_scale must be None unless the KV cache is float8_e4m3fn")
+        if fp8:
+            named.update(k_scale=k_scale, v_scale=v_scale)
+        for name, t in named.items():
+            if t.device != q.device:
+                raise ValueError(f"Expected {name} on {q.device}, got {t.device}")
+        want_q = (self.batch, self.heads, self.dim)
+        if tuple(q.shape) != want_q:
+            raise ValueError(f"Expected q.shape {want_q}, got {tuple(q.shape)}")
+        if k.dim() != 4 or k.shape[0] != self.batch or tuple(k.shape[2:]) != (self.heads_kv, self.dim):
+            raise ValueError(f"Expected k.shape ({self.batch}, N_kv, {self.heads_kv}, {self.dim}), got {tuple(k.shape)}")
+        if tuple(v.shape) != tuple(k.shape):
+            raise ValueError(f"Expected v.shape {tuple(k.shape)}, got {tuple(v.shape)}")
+        if k.shape[1] > self.seqlen_kv:
+            raise ValueError(f"k holds {k.shape[1]} tokens per sequence but the op was built for seqlen_kv={self.seqlen_kv}")
+        for name, t in named.items():
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous")
+        if fp8:
+            for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+                if tuple(t.shape) != tuple(k.shape[:3]):
+                    raise ValueError(f"Expected {name}.shape {tuple(k.shape[:3])}, got {tuple(t.shape)}")
+
+    def observe_call(self, real_seqlen_kv: int, kv_dtype: torch.dtype) -> None:
+        """Record the context length of a call so that ``eval_roofline`` prices the bytes actually addressed."""
+        self._seen_call = {
+            "sum_len": int(real_seqlen_kv) * self.batch, "sum_pages": 0,
+            "kv_bytes": torch.empty((), dtype=kv_dtype).element_size(), "fp8": kv_dtype == FP8,
+        }
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+                v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        self._validate_call(q, k, v, k_scale, v_scale)
+        self.dtype = q.dtype
+        real_seqlen_kv = k.shape[1]
+        kernel = self._get_kernel((q, k, v, k_scale, v_scale), q.dtype, k.dtype)
+        if k_scale is None:
+            return kernel(q, k, v, real_seqlen_kv)
+        return kernel(q, k, v, real_seqlen_kv, k_scale, v_scale)

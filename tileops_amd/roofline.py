@@ -75,3 +75,24 @@ def gqa_decode_paged_roofline(op: Optional[Any] = None, **kwargs: Any) -> tuple[
     b = algorithmic_bytes(sum_len=seen["sum_len"], sum_pages=seen["sum_pages"], batch=batch, q_len=q_len, heads=heads,
                           heads_kv=heads_kv, dim=dim, q_bytes=q_bytes, kv_bytes=seen["kv_bytes"], fp8_scales=seen["fp8"])
     return algorithmic_flops(sum_len=seen["sum_len"], q_len=q_len, heads=heads, dim=dim), b["total"]
+
+
+def gqa_decode_roofline(op: Optional[Any] = None, **kwargs: Any) -> tuple[int, int]:
+    """Contiguous-cache GQA decode: the reference formula (src/tileops/perf/formulas.py:668-687) from shapes;
+    once the op has seen a call, the tokens it actually addressed instead of the allocated ``seqlen_kv``."""
+    d = _fields(op, kwargs)
+    if "q_shape" in d:
+        batch, heads, dim = d["q_shape"]
+        _, seqlen_kv, heads_kv, _ = d["kv_shape"]
+    else:
+        batch, heads, heads_kv, seqlen_kv, dim = d["batch"], d["heads"], d["heads_kv"], d["seqlen_kv"], d["dim"]
+    q_bytes = _itemsize(d.get("dtype") or d.get("dtypes") or "float16")
+    seen = d.get("_seen_call")
+    if seen is None:
+        flops = 4 * batch * heads * seqlen_kv * dim
+        q_elems = batch * heads * dim
+        kv_elems = batch * seqlen_kv * heads_kv * dim
+        return int(flops), int((q_elems + 2 * kv_elems + q_elems) * q_bytes)
+    b = algorithmic_bytes(sum_len=seen["sum_len"], sum_pages=0, batch=batch, q_len=1, heads=heads, heads_kv=heads_kv,
+                          dim=dim, q_bytes=q_bytes, kv_bytes=seen["kv_bytes"], fp8_scales=seen["fp8"])
+    return algorithmic_flops(sum_len=seen["sum_len"], q_len=1, heads=heads, dim=dim), b["total"] - 4 * batch
