@@ -764,19 +764,25 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
 // Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
 //   lse = log2 sum_s 2^(lse_s - max) + max ; O = sum_s 2^(lse_s - lse) * O_s   (reference combine,
 //   src/tileops/kernels/attention/gqa_decode_paged.py:344-374), on fp32 partials.
-// One wave per (sequence, kv head, query row): lane i fetches the LSE of the i-th partition of the sequence,
-// the weights are formed with two wave reductions, then every lane accumulates two head elements over the
-// partitions with independent loads.  grid (heads_kv*rows, batch), 64 threads.
-template <typename QT>
-__global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix) {
-  const int b = blockIdx.y, row_all = blockIdx.x, lane = threadIdx.x;
+// One workgroup of four waves per (sequence, kv head, query row).  Every wave forms the maximum and the sum of
+// weights over all partitions of the sequence (lane i fetches the LSE of partition i, two wave reductions per 64);
+// the weighted sum of the partial rows is split over the waves (wave w takes partitions w, w+4, ...), eight
+// independent row loads in flight per wave, every lane two head elements; the four sums meet in LDS.  With at
+// most eight partitions wave 0 works alone and the others leave at once.  A single
+// sequence spread over hundreds of partitions (batch-1 long-context decode) is then merged in a few load round
+// trips instead of one per partition.  grid (heads_kv*rows, batch), 64*kCombineWaves threads; the launcher takes the
+// one-wave instance when the average sequence spans at most eight partitions.
+template <typename QT, int kCombineWaves>
+__global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix) {
+  __shared__ f32x2 red[kCombineWaves][64];
+  const int b = blockIdx.y, row_all = blockIdx.x, lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
   const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
   const int s = r / p.group, gi = r - s * p.group;
   uint32_t* op = (uint32_t*)((uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) + lane;
   const int4 rec = ((const int4*)ws_prefix)[b];  // the only load everything else depends on
   const int p_first = rec.y, p_last = rec.z;
   if (p_first < 0) {  // empty sequence: the attention kernel never visits it
-    *op = 0;
+    if (wave == 0) *op = 0;
     return;
   }
   if (p_first == p_last) return;  // one wave covered the whole sequence and wrote the output itself
@@ -786,51 +792,67 @@ __global__ __launch_bounds__(64) void paged_decode_mfma_combine_kernel(const Dec
   const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
   const int n = p_last - p_first + 1;
   auto slot_of = [&](int pp) { return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all; };
-  float acc0 = 0.f, acc1 = 0.f, W = 0.f, M = -INFINITY;
-  for (int base = 0; base < n; base += 64) {  // a sequence seldom spans more than a handful of partitions
+  auto owns_tiles = [&](int pp) { return !gaps || part_begin(pp + 1, T, NP) > part_begin(pp, T, NP); };
+  constexpr int PRE = 8;
+  // up to eight partitions (the usual case when many sequences share the chip): one wave does it all
+  const int nw = n <= PRE ? 1 : kCombineWaves;
+  if (wave >= nw) return;
+  // this wave's first eight partial rows go out together with the LSEs, before any weight is known
+  f32x2 rows[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; i++) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + wave + nw * i, p_last)) * kD + 2 * lane);
+  // lane i keeps the LSE of partition i of the first 64 (all of them, as a rule); further ones are re-read
+  const float lse0 = (p_first + lane <= p_last && owns_tiles(p_first + lane)) ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
+  float M = lse0;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) M = fmaxf(M, __shfl_xor(M, m, 64));
+  for (int base = 64; base < n; base += 64) {
     const int pp = p_first + base + lane;
-    bool valid = pp <= p_last;
-    if (valid && gaps) valid = part_begin(pp + 1, T, NP) > part_begin(pp, T, NP);
-    const float lse = valid ? p.part_lse[slot_of(pp)] : -INFINITY;
-    // the first eight partials are fetched together with the LSEs, before the weights are known
-    constexpr int PRE = 8;
-    f32x2 pre_v[PRE];
+    float lse = (pp <= p_last && owns_tiles(pp)) ? p.part_lse[slot_of(pp)] : -INFINITY;
 #pragma unroll
-    for (int i = 0; i < PRE; i++) {
-      const int pi = min(p_first + base + i, p_last);
-      pre_v[i] = *(const f32x2*)(p.part_o + slot_of(pi) * kD + 2 * lane);
+    for (int m = 1; m < 64; m <<= 1) lse = fmaxf(lse, __shfl_xor(lse, m, 64));
+    M = fmaxf(M, lse);
+  }
+  const float w0 = (M != -INFINITY && lse0 != -INFINITY) ? fast_exp2(lse0 - M) : 0.f;  // weight of partition `lane`
+  float W = w0;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) W += __shfl_xor(W, m, 64);
+  if (M != -INFINITY) {
+    for (int base = 64; base < n; base += 64) {  // second pass over the (now cached) LSEs
+      const int pp = p_first + base + lane;
+      float w = (pp <= p_last && owns_tiles(pp)) ? fast_exp2(p.part_lse[slot_of(pp)] - M) : 0.f;
+#pragma unroll
+      for (int m = 1; m < 64; m <<= 1) w += __shfl_xor(w, m, 64);
+      W += w;
     }
-    float m_chunk = lse;
+  }
+  float acc0 = 0.f, acc1 = 0.f;
+  if (W > 0.f) {
+    for (int i0 = 0; wave + nw * i0 < n; i0 += PRE) {
+      float wt[PRE];
 #pragma unroll
-    for (int m = 1; m < 64; m <<= 1) m_chunk = fmaxf(m_chunk, __shfl_xor(m_chunk, m, 64));
-    const float M_new = fmaxf(M, m_chunk);
-    if (M_new == -INFINITY) continue;
-    const float rescale = fast_exp2(M - M_new);  // 0 on the first chunk (M = -inf)
-    acc0 *= rescale;
-    acc1 *= rescale;
-    W *= rescale;
-    M = M_new;
-    const float w_lane = valid ? fast_exp2(lse - M) : 0.f;
-    float w_sum = w_lane;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) w_sum += __shfl_xor(w_sum, m, 64);
-    W += w_sum;
-    const int cnt = min(64, n - base);
-#pragma unroll
-    for (int i = 0; i < PRE; i++) {
-      const float w = __shfl(w_lane, i, 64);  // 0 for lanes past the last partition
-      if (w != 0.f) {
-        acc0 = fmaf(w, pre_v[i][0], acc0);
-        acc1 = fmaf(w, pre_v[i][1], acc1);
+      for (int i = 0; i < PRE; i++) {
+        const int idx = wave + nw * (i0 + i), pp = p_first + idx;  // wave-uniform
+        if (idx < 64) wt[i] = __shfl(w0, idx, 64);
+        else wt[i] = (pp <= p_last && owns_tiles(pp)) ? fast_exp2(p.part_lse[slot_of(pp)] - M) : 0.f;
+        if (i0 > 0) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(pp, p_last)) * kD + 2 * lane);
       }
+#pragma unroll
+      for (int i = 0; i < PRE; i++)
+        if (wt[i] != 0.f) {  // an unwritten slot may hold anything, NaN included
+          acc0 = fmaf(wt[i], rows[i][0], acc0);
+          acc1 = fmaf(wt[i], rows[i][1], acc1);
+        }
     }
-    for (int i = PRE; i < cnt; i++) {
-      const float w = __shfl(w_lane, i, 64);
-      if (w != 0.f) {
-        const f32x2 v = *(const f32x2*)(p.part_o + slot_of(p_first + base + i) * kD + 2 * lane);
-        acc0 = fmaf(w, v[0], acc0);
-        acc1 = fmaf(w, v[1], acc1);
-      }
+  }
+  if (nw > 1) {  // uniform over the workgroup: either every wave is here or only wave 0 exists
+    red[wave][lane] = f32x2{acc0, acc1};
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int w = 1; w < kCombineWaves; w++) {
+      acc0 += red[w][lane][0];
+      acc1 += red[w][lane][1];
     }
   }
   const float inv = W > 0.f ? 1.0f / W : 0.f;
@@ -864,7 +886,11 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
   if (skip_combine) return nullptr;
-  hipLaunchKernelGGL(paged_decode_mfma_combine_kernel<QT>, dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
+  // four waves per row when sequences span many partitions on average, one otherwise (fewer waves to launch)
+  if ((int64_t)p.n_parts > 8 * (int64_t)p.batch)
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), dim3(p.heads_kv * p.rows, p.batch), dim3(256), 0, s, p, ws_prefix);
+  else
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }

@@ -1,0 +1,299 @@
+"""Manifest-driven benchmark of the ops, reporting in the reference's formats.
+
+Takes the place of the reference's benchmark plumbing for these ops (benchmarks/ops/attention/
+bench_gqa_decode_paged.py:150-210 and bench_gqa_decode.py drive the manifest workloads; benchmarks/report.py:117-262
+collects records and dumps ``profile_run.log``; benchmarks/conftest.py:52-136 attaches ``<tag>_<metric>``
+properties to the JUnit XML).  This runner needs no pytest plugin: it walks the manifest, times every workload
+and writes both artefacts itself.
+
+    python -m tileops_amd.perf.manifest_bench [--op NAME] [--label SUBSTR] [--steps N] [--out DIR]
+
+Per workload and implementation (tag) it records ``latency_ms`` (median device time of one call, HIP events, the
+L2/MALL flushed between calls -- the methodology of benchmarks/timing.py:546-585), ``tflops`` and
+``bandwidth_tbs`` from the op's ``eval_roofline()`` after it has seen the call, and ``hbm_frac`` = bandwidth over
+the 8 TB/s peak.  ``device_busy_ms`` (sum of kernel durations) is taken from the torch profiler when it delivers
+device events, otherwise left out.  Baseline tag ``torch_sdpa``: ``F.scaled_dot_product_attention`` on the same
+device for the contiguous op (no FlashInfer / AITER build is importable in this image; the tag slot is there).
+"""
+
+from __future__ import annotations
+
+import argparse
+import statistics
+import subprocess
+import sys
+import xml.etree.ElementTree as ET
+from datetime import datetime
+from pathlib import Path
+from typing import Any, Callable, Optional
+
+import torch
+
+from .. import native
+from ..manifest import load_manifest
+from ..ops import (
+    GroupedQueryAttentionDecodePagedWithKVCacheFwdOp, GroupedQueryAttentionDecodeWithKVCacheFwdOp,
+    GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp,
+)
+from ..workloads import FP8, GroupedQueryAttentionDecodePagedWorkload, PagedDecodeConfig, gen_paged_inputs, quantize_kv_per_token
+
+HBM_PEAK_TBS = 8.0
+_DT = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float8_e4m3fn": FP8}
+
+
+class BenchmarkReport:
+    """Records per op and tag, dumped as the markdown log the reference leaves behind (report.py:117-262)."""
+
+    def __init__(self) -> None:
+        self.records: dict[str, list[dict]] = {}
+
+    def record(self, op_name: str, params: dict, result: dict, tag: str = "tileops", config: Optional[dict] = None) -> None:
+        entry = {"params": params, "result": result, "tag": tag}
+        if config:
+            entry["config"] = config
+        self.records.setdefault(op_name, []).append(entry)
+
+    @staticmethod
+    def _environment() -> list[str]:
+        lines = [f"- **Torch version**: {torch.__version__}", f"- **HIP version (torch)**: {torch.version.hip or 'N/A'}"]
+        if torch.cuda.is_available():
+            props = torch.cuda.get_device_properties(0)
+            lines.append(f"- **GPU model**: {props.name} ({getattr(props, 'gcnArchName', '?')}, {props.multi_processor_count} CUs)")
+        else:
+            lines.append("- **GPU model**: N/A (no device)")
+        try:
+            out = subprocess.run(["rocm-smi", "--showdriverversion"], capture_output=True, text=True, timeout=10).stdout
+            driver = next((ln.split(":")[-1].strip() for ln in out.splitlines() if "Driver version" in ln), "N/A")
+        except (FileNotFoundError, subprocess.TimeoutExpired):
+            driver = "N/A"
+        lines.append(f"- **Driver version**: {driver}")
+        return lines
+
+    def dump(self, path: Path) -> None:
+        if not self.records:
+            return
+        lines = ["# TileOPs Benchmark Report", f"Generated: {datetime.now().strftime('%Y-%m-%d %H:%M:%S')}", "",
+                 "## Environment", "", *self._environment(), ""]
+        default_keys = ["device_busy_ms", "latency_ms", "gap_ms", "n_kernels", "tflops", "bandwidth_tbs"]
+        for name, entries in self.records.items():
+            lines += [f"## {name}", ""]
+            keys = list(default_keys)
+            for e in entries:
+                keys += [k for k in e["result"] if k not in keys]
+            by_tag: dict[str, list[dict]] = {}
+            for e in entries:
+                by_tag.setdefault(e["tag"], []).append(e)
+            for tag, group in by_tag.items():
+                lines += [f"### {tag}", ""]
+                pkeys = list(group[0]["params"])
+                has_cfg = any("config" in e for e in group)
+                header = pkeys + keys + (["config"] if has_cfg else [])
+                lines.append("| " + " | ".join(header) + " |")
+                lines.append("| " + " | ".join(["---"] * len(header)) + " |")
+                for e in group:
+                    row = [str(e["params"].get(k, "")) for k in pkeys]
+                    for k in keys:
+                        val = e["result"].get(k)
+                        row.append("N/A" if val is None else (f"{val:.4f}" if isinstance(val, (int, float)) and not isinstance(val, bool) else str(val)))
+                    if has_cfg:
+                        row.append(str(e.get("config") or ""))
+                    lines.append("| " + " | ".join(row) + " |")
+                lines.append("")
+        path.write_text("\n".join(lines) + "\n", encoding="utf-8")
+
+
+def _prop(value: Any) -> str:
+    """benchmarks/conftest.py:36-47: significant digits, not fixed decimals."""
+    if isinstance(value, (bool, int)):
+        return str(value)
+    if isinstance(value, float):
+        return str(int(value)) if value.is_integer() else f"{value:.6g}"
+    return str(value)
+
+
+class _Flusher:
+    """Evicts L2 and the memory-side cache between timed calls: a 512 MiB write followed by a 512 MiB read."""
+
+    def __init__(self, device: torch.device) -> None:
+        self.w = torch.empty(512 << 20, dtype=torch.uint8, device=device)
+        self.r = torch.ones(128 << 20, dtype=torch.int32, device=device)
+        self.i = 0
+
+    def __call__(self) -> None:
+        self.i += 1
+        self.w.fill_(self.i & 255)
+        self.r.max()
+
+
+def _time(fn: Callable[[], Any], flush: _Flusher, steps: int, warmup: int = 3) -> float:
+    for _ in range(warmup):
+        fn()
+    ts = []
+    for _ in range(steps):
+        flush()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        ts.append(a.elapsed_time(b))
+    return statistics.median(ts)
+
+
+def _device_busy(fn: Callable[[], Any]) -> tuple[Optional[float], Optional[int]]:
+    """(sum of kernel durations in ms, number of kernels) of one call, from the torch profiler; (None, None) if
+    the profiler delivers no device events on this build."""
+    try:
+        from torch.profiler import ProfilerActivity, profile
+        fn()
+        torch.cuda.synchronize()
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            fn()
+            torch.cuda.synchronize()
+        evs = [e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA]
+        if not evs:
+            return None, None
+        return sum(e.device_time for e in evs) / 1e3, len(evs)
+    except Exception:  # noqa: BLE001 - the profiler is optional evidence, never a reason to fail a benchmark
+        return None, None
+
+
+def _result(op: Any, latency_ms: float, busy: tuple[Optional[float], Optional[int]]) -> dict:
+    flops, nbytes = op.eval_roofline()
+    res = {"latency_ms": latency_ms, "tflops": flops / latency_ms / 1e9, "bandwidth_tbs": nbytes / latency_ms / 1e9}
+    res["hbm_frac"] = res["bandwidth_tbs"] / HBM_PEAK_TBS
+    if busy[0] is not None:
+        res["device_busy_ms"], res["n_kernels"] = busy[0], busy[1]
+        res["gap_ms"] = max(latency_ms - busy[0], 0.0)
+    return res
+
+
+def _paged_case(row: dict, dtype: torch.dtype, device: torch.device, multi: bool):
+    qs, (n_kv, heads_kv, dim) = row["q_shape"], row["kv_shape"]
+    batch, heads = qs[0], qs[-2]
+    q_len = qs[1] if multi else 1
+    page = row["page_size"]
+    kv_dtype = _DT[row.get("kv_dtype", str(dtype).removeprefix("torch."))]
+    kw = dict(sm_scale=row.get("sm_scale"), softcap=row.get("softcap"))
+    if multi:
+        op = GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp(batch, q_len, heads, heads_kv, n_kv, dim, page, **kw)
+    else:
+        op = GroupedQueryAttentionDecodePagedWithKVCacheFwdOp(batch, heads, heads_kv, n_kv, dim, page, **kw)
+    if "seqlen_range" in row:  # ragged lengths over a shared pool with a permuted block table
+        cfg = PagedDecodeConfig(row["label"], batch, heads, heads_kv, dim, page, n_kv // page, tuple(row["seqlen_range"]),
+                                q_len=q_len, dtype=dtype, kv_dtype=kv_dtype, seed=row.get("seed", 0))
+        inp = gen_paged_inputs(cfg, device)
+        args = (inp.q, inp.k, inp.v, inp.real_seqlen_kv, inp.block_table) + ((inp.k_scale, inp.v_scale) if inp.k_scale is not None else ())
+        lens = inp.real_seqlen_kv
+    else:  # the reference's generator: page-multiple random lengths, identity table
+        wl = GroupedQueryAttentionDecodePagedWorkload(batch, heads, heads_kv, n_kv, dim, page, dtype, **kw)
+        args = wl.gen_inputs(device)
+        lens = args[3]
+    op.observe_call(lens, kv_dtype)
+    return op, args, None
+
+
+def _contiguous_case(row: dict, dtype: torch.dtype, device: torch.device):
+    (batch, heads, dim), (_, n_kv, heads_kv, _) = row["q_shape"], row["kv_shape"]
+    kv_dtype = _DT[row.get("kv_dtype", str(dtype).removeprefix("torch."))]
+    op = GroupedQueryAttentionDecodeWithKVCacheFwdOp(batch, heads, heads_kv, n_kv, dim, sm_scale=row.get("sm_scale"),
+                                                     softcap=row.get("softcap"))
+    q = torch.randn(batch, heads, dim, device=device, dtype=dtype)
+    k = torch.randn(batch, n_kv, heads_kv, dim, device=device, dtype=dtype)
+    v = torch.randn(batch, n_kv, heads_kv, dim, device=device, dtype=dtype)
+    baseline = None
+    if kv_dtype == FP8:
+        k8, ks = quantize_kv_per_token(k.reshape(-1, heads_kv, dim))
+        v8, vs = quantize_kv_per_token(v.reshape(-1, heads_kv, dim))
+        args = (q, k8.reshape(k.shape), v8.reshape(v.shape), ks.reshape(batch, n_kv, heads_kv), vs.reshape(batch, n_kv, heads_kv))
+    else:
+        args = (q, k, v)
+        if not row.get("softcap"):
+            import torch.nn.functional as F
+            qb, kb, vb = q.unsqueeze(2), k.transpose(1, 2), v.transpose(1, 2)  # [B,H,1,D], [B,Hkv,N,D]
+
+            def baseline():
+                return F.scaled_dot_product_attention(qb, kb, vb, scale=op.sm_scale, enable_gqa=True)
+    op.observe_call(n_kv, kv_dtype)
+    return op, args, baseline
+
+
+_CASES = {
+    "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp": lambda r, d, dev: _paged_case(r, d, dev, False),
+    "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp": lambda r, d, dev: _paged_case(r, d, dev, True),
+    "GroupedQueryAttentionDecodeWithKVCacheFwdOp": _contiguous_case,
+}
+
+
+def main(argv: Optional[list[str]] = None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--op", default=None, help="only this op (class name)")
+    ap.add_argument("--label", default=None, help="only workloads whose label contains this")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--max-kv-gib", type=float, default=8.0, help="skip workloads whose K+V exceed this")
+    ap.add_argument("--out", default="manifest_bench_out", help="directory for junit.xml and profile_run.log")
+    args = ap.parse_args(argv)
+    device = torch.device("cuda", 0)
+    native.require_gfx950(device)
+    out_dir = Path(args.out)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    report, flush = BenchmarkReport(), _Flusher(device)
+    suite = ET.Element("testsuite", name="tileops_amd.manifest_bench")
+    n = 0
+    for op_name, entry in load_manifest().items():
+        if op_name not in _CASES or (args.op and args.op != op_name):
+            continue
+        for row in entry["workloads"]:
+            if args.label and args.label not in row["label"]:
+                continue
+            for dname in row["dtypes"]:
+                dtype = _DT[dname]
+                kv_elems = 2
+                for s in row["kv_shape"]:
+                    kv_elems *= s
+                if kv_elems * 2 / 2**30 > args.max_kv_gib:
+                    print(f"skip {op_name} {row['label']} {dname}: K+V of {kv_elems * 2 / 2**30:.1f} GiB", flush=True)
+                    continue
+                torch.manual_seed(1235)
+                op, inputs, baseline = _CASES[op_name](row, dtype, device)
+                call = lambda: op(*inputs)  # noqa: E731
+                lat = _time(call, flush, args.steps)
+                res = _result(op, lat, _device_busy(call))
+                kernel = next(iter(op.iter_kernels()), None) if hasattr(op, "iter_kernels") else None
+                params = {"label": row["label"], "q_shape": tuple(row["q_shape"]), "kv_shape": tuple(row["kv_shape"]), "dtype": dname,
+                          "kv_dtype": row.get("kv_dtype", dname)}
+                if "page_size" in row:
+                    params["page_size"] = row["page_size"]
+                report.record(op_name, params, res, "tileops", getattr(kernel, "config", None))
+                case = ET.SubElement(suite, "testcase", classname=op_name, name=f"{row['label']}-{dname}", time=f"{lat / 1e3:.6f}")
+                props = ET.SubElement(case, "properties")
+                ET.SubElement(props, "property", name="op", value=op_name)
+                ET.SubElement(props, "property", name="op_module", value=type(op).__module__)
+                for key, val in res.items():
+                    ET.SubElement(props, "property", name=f"tileops_{key}", value=_prop(val))
+                line = f"{op_name[:40]:40s} {row['label']:28s} {dname:9s} {lat * 1e3:9.1f} us  {res['bandwidth_tbs']:.2f} TB/s ({100 * res['hbm_frac']:.1f}%)"
+                if baseline is not None:
+                    bl = _time(baseline, flush, max(args.steps // 2, 3))
+                    flops, nbytes = op.eval_roofline()
+                    bres = {"latency_ms": bl, "tflops": flops / bl / 1e9, "bandwidth_tbs": nbytes / bl / 1e9}
+                    report.record(op_name, params, bres, "torch_sdpa")
+                    ET.SubElement(props, "property", name="baseline_tag", value="torch_sdpa")
+                    for key, val in bres.items():
+                        ET.SubElement(props, "property", name=f"torch_sdpa_{key}", value=_prop(val))
+                        ET.SubElement(props, "property", name=f"baseline_{key}", value=_prop(val))
+                    ET.SubElement(props, "property", name="torch_sdpa_ratio", value=f"{bl / lat:.4f}")
+                    ET.SubElement(props, "property", name="baseline_ratio", value=f"{bl / lat:.4f}")
+                    line += f"   torch_sdpa {bl * 1e3:9.1f} us (x{bl / lat:.2f})"
+                print(line, flush=True)
+                n += 1
+                del op, inputs, baseline, call
+                torch.cuda.empty_cache()
+    suite.set("tests", str(n))
+    ET.ElementTree(suite).write(out_dir / "junit.xml", encoding="utf-8", xml_declaration=True)
+    report.dump(out_dir / "profile_run.log")
+    print(f"{n} workloads -> {out_dir}/junit.xml, {out_dir}/profile_run.log")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
