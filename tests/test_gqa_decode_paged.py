@@ -408,3 +408,61 @@ def test_tune_picks_a_config_and_stays_correct():
     _check_reference_style(op, wl, inputs)
     kernel = next(iter(op.built_kernels(next(iter(op._kernel_roles))).values()))
     assert kernel.config in kernel.autotune_configs
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("fp8", [False, True])
+def test_more_than_64_sequences_with_empty_ones_in_between(kernel_key, fp8):
+    """Batch 150: the per-wave caches of sequence lengths hold 64 entries and are refilled while a wave walks the
+    tile stream; empty sequences sit at the refill boundaries, at the start and at the end."""
+    require_gfx950()
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(1, 400, (150,), generator=g).tolist()
+    for b in (0, 63, 64, 65, 127, 128, 149):
+        lens[b] = 0
+    lens[66] = 3000
+    case = _ragged_case(len(lens), 16, 4, 128, 32, lens, torch.bfloat16, fp8=fp8, seed=33)
+    op = PagedOp(len(lens), 16, 4, case[1].shape[0], 128, 32)
+    if not _serves(op, kernel_key, torch.bfloat16, fp8):
+        pytest.skip(f"{kernel_key} does not serve this shape")
+    _force(op, kernel_key)
+    out = _run_and_compare(op, case, 32, 3e-2 if fp8 else 2e-2)
+    assert (out[[0, 63, 64, 65, 127, 128, 149]] == 0).all()
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_graph_capture_and_replay_with_changing_cache_contents(fp8):
+    """The call captured in a HIP graph and replayed: every replay, with eager work and synchronisation in between
+    and new K/V values written into the same pool, must equal the eager result on the same contents."""
+    require_gfx950()
+    lens = [900, 33, 2048, 5, 1500, 64]
+    case = _ragged_case(len(lens), 32, 8, 128, 64, lens, torch.bfloat16, fp8=fp8, seed=9)
+    dev = [None if t is None else t.to(DEV) for t in case]
+    args = dev[:5] if not fp8 else dev
+    op = PagedOp(len(lens), 32, 8, case[1].shape[0], 128, 64)
+    eager0 = op(*args)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            op(*args)  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = op(*args)
+    for it in range(4):
+        if it:  # new contents in place: same pointers, different values
+            if fp8:  # flip signs: the NaN poison of unaddressed tokens stays where it is
+                args[1].view(torch.uint8).bitwise_xor_(0x80)
+                args[6].mul_(1.0 + 0.25 * it)
+            else:
+                args[1].mul_(-0.5)
+                args[2].mul_(1.0 + 0.25 * it)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = op(*args)
+        torch.cuda.synchronize()
+        assert torch.isfinite(eager).all()
+        assert torch.equal(out_g, eager), f"replay {it} differs from the eager call"
+        assert torch.equal(eager, eager0) == (it == 0)
