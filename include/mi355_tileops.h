@@ -130,6 +130,41 @@ int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k
                      int causal, int num_split, int kernel, void* hip_stream);
 
 /*
+ * Packed GQA prefill chunk with paged KV-cache append: one call = one forward of
+ * GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp (src/tileops/ops/attention/gqa.py:1072-1140 ->
+ * GQAPrefillPagedWithKVCacheFwdKernel / GQAPrefillPagedWithFP8KVCacheFwdKernel,
+ * src/tileops/kernels/attention/gqa_fwd.py:600-1000 and :1005-1460).  Fused RoPE (the third reference kernel) is
+ * not served.
+ *
+ *   q              [total_q, heads, dim] q_dtype: the chunks of all sequences packed; sequence b owns rows
+ *                  [cu_seqlens_q[b], cu_seqlens_q[b+1])
+ *   k_new, v_new   [total_q, heads_kv, dim] q_dtype: keys/values of the same rows
+ *   k_pages,
+ *   v_pages        [n_phys_tokens, heads_kv, dim] cache_dtype (q_dtype or fp8): the page pool.  The chunk is appended at
+ *                  logical positions cache_seqlens[b] + i (16-bit: copied; fp8: clamp(x / scale, +-448) -> e4m3fn,
+ *                  gqa_fwd.py:1059-1061, :1124-1168)
+ *   k_scale,
+ *   v_scale        [1] fp32 per-tensor dequantisation scales (x = fp8 * scale); read only with an fp8 cache
+ *   cu_seqlens_q   [batch + 1] int32;  cache_seqlens [batch] int32: context length of each sequence before the append
+ *   block_table    [batch, >= ceil((cache_seqlens[b] + q_len_b) / page_size)] int32, row stride bt_row_stride
+ *   out            [total_q, heads, dim] q_dtype
+ *   max_seqlen_q   upper bound of the chunk lengths (sizes the launch; a longer chunk would lose its last rows)
+ *   causal         query i of a chunk sees the old tokens and chunk tokens j <= i (gqa_fwd.py:1247-1256); 0: all of them
+ * Attention runs over the dequantised old tokens and the *unquantised* chunk (as the reference: :1180-1245): with an fp8
+ * cache that is two passes (pages, then k_new/v_new) whose fp32 results are merged by log-sum-exp.
+ * Sequences with an empty chunk produce no output rows and append nothing.
+ */
+int mi355_gqa_prefill_paged_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
+                                      int page_size, int64_t max_pages_per_req, int q_dtype, int cache_dtype, int kernel,
+                                      size_t* workspace_bytes);
+int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new, void* k_pages, void* v_pages,
+                            const float* k_scale, const float* v_scale, const int32_t* cu_seqlens_q,
+                            const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,
+                            void* workspace, size_t workspace_bytes, int batch, int max_seqlen_q, int64_t total_q, int heads,
+                            int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype, int cache_dtype,
+                            float sm_scale, float softcap, int causal, int kernel, void* hip_stream);
+
+/*
  * Index-probe: materialise the logical KV rows a decode call would read, with the same device page
  * arithmetic the attention kernels use.  dense_out [batch, max_len, heads_kv * dim] elem_bytes-wide
  * elements; rows t >= seqlens[b] are left untouched.  Lets a test compare the gather bit-for-bit with

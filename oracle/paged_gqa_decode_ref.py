@@ -15,6 +15,9 @@ Parity status of each function (how it is pinned, without importing the referenc
 * ``ref_gqa_decode_contiguous`` pinned against SDPA and the paged oracle with an identity table.
 * ``quantize_kv_per_token``     pinned against the C codec in ``oracle/fp8_e4m3fn.c`` and torch's fp8 cast.
 * causal chunk mask             pinned by "query i of a chunk == single-token decode at length len-S_q+i+1".
+* ``ref_gqa_prefill_paged``     pinned against SDPA per sequence (explicit boolean mask), against "row i of a chunk ==
+                                single-token decode over old tokens + chunk[:i+1]" through the pinned decode oracle,
+                                and, for the append, against a per-token loop over ``physical_pos`` and torch's fp8 cast.
 
 The exact floating-point bits of the reference's TileLang-generated CUDA kernels are not reproducible here
 (TileLang is absent); the reference itself defines correctness against this torch program within tolerance.
@@ -242,3 +245,79 @@ def reference_roofline(
     kv_elems = seqlen_kv * heads_kv * dim
     meta = batch * 4 + batch * max(1, (seqlen_kv + page_size - 1) // page_size) * 4
     return int(flops), int((q_elems + 2 * kv_elems + q_elems) * elem_bytes + meta)
+
+
+def quantize_per_tensor(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """``clamp(x / scale, -448, 448)`` cast to e4m3fn (round to nearest even): the append of the reference's FP8 paged
+    prefill kernel, src/tileops/kernels/attention/gqa_fwd.py:1059-1061; expectation of its test,
+    tests/ops/attention/test_gqa_prefill_paged.py:402-405."""
+    return (x.float() / scale.float().reshape(())).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+
+
+def ref_gqa_prefill_paged(
+    q: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    k_scale: torch.Tensor,
+    v_scale: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cache_seqlens: torch.Tensor,
+    block_table: torch.Tensor,
+    *,
+    page_size: int,
+    is_causal: bool = True,
+    sm_scale: Optional[float] = None,
+    softcap: float = 0.0,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Packed prefill chunk over a paged cache: ``(o [total_q,H,D], k_pages_after, v_pages_after)``.
+
+    Restates ``_gqa_prefill_paged_ref`` and the append checks of the reference's test
+    (tests/ops/attention/test_gqa_prefill_paged.py:76-117, :301-313, :398-415): per sequence, attention in fp32 over
+    ``cat(old tokens, chunk)`` with ``kv_pos <= old_len + i`` when causal; the old tokens of an FP8 cache are
+    dequantised as ``(fp8.float() * scale).to(q.dtype)`` (:347-348; kernel: gqa_fwd.py:1063-1065), the chunk's own
+    tokens enter unquantised; the chunk is written to logical positions ``old_len + i`` (copied, or quantised per
+    tensor for an FP8 cache); nothing else in the pool changes.
+    """
+    total_q, H, D = q.shape
+    H_kv = k_new.shape[1]
+    G = H // H_kv
+    scale = D ** -0.5 if sm_scale is None else sm_scale
+    fp8 = k_pages.dtype == torch.float8_e4m3fn
+    k_after, v_after = k_pages.clone(), v_pages.clone()
+    out = torch.zeros(total_q, H, D, dtype=q.dtype)
+    batch = cache_seqlens.shape[0]
+    for b in range(batch):
+        q0, q1 = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1])
+        q_len, old_len = q1 - q0, int(cache_seqlens[b])
+        if q_len == 0:
+            continue
+        idx = torch.tensor([physical_pos(block_table, b, t, page_size) for t in range(old_len)], dtype=torch.long)
+        k_old, v_old = k_pages[idx], v_pages[idx]
+        if fp8:
+            k_old = (k_old.float() * k_scale.float().reshape(())).to(q.dtype)
+            v_old = (v_old.float() * v_scale.float().reshape(())).to(q.dtype)
+        k_all = torch.cat([k_old.to(q.dtype), k_new[q0:q1]], 0).float()
+        v_all = torch.cat([v_old.to(q.dtype), v_new[q0:q1]], 0).float()
+        total_len = old_len + q_len
+        qg = q[q0:q1].float().reshape(q_len, H_kv, G, D)
+        scores = torch.einsum("sjgd,njd->jgsn", qg, k_all) * scale
+        if softcap > 0:
+            scores = softcap * torch.tanh(scores / softcap)
+        if is_causal:
+            q_pos = torch.arange(q_len)[:, None] + old_len
+            kv_pos = torch.arange(total_len)[None, :]
+            scores = scores.masked_fill(~(kv_pos <= q_pos), float("-inf"))
+        probs = torch.softmax(scores, dim=-1).nan_to_num()
+        o = torch.einsum("jgsn,njd->sjgd", probs, v_all)
+        out[q0:q1] = o.reshape(q_len, H, D).to(q.dtype)
+        for i in range(q_len):
+            pos = physical_pos(block_table, b, old_len + i, page_size)
+            if fp8:
+                k_after[pos] = quantize_per_tensor(k_new[q0 + i], k_scale)
+                v_after[pos] = quantize_per_tensor(v_new[q0 + i], v_scale)
+            else:
+                k_after[pos] = k_new[q0 + i]
+                v_after[pos] = v_new[q0 + i]
+    return out, k_after, v_after

@@ -89,12 +89,22 @@ int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_s
   return MI355_OK;
 }
 
+// What a prefill chunk adds to a decode call (all zero for the decode entry points).
+struct Extras {
+  const int32_t* cu_q = nullptr;
+  int len_excludes_new = 0;
+  const int32_t* kv_starts = nullptr;
+  int scale_per_tensor = 0;
+  float* final_o = nullptr;
+  float* final_lse = nullptr;
+};
+
 // One decode call, paged (block_table/seqlens given) or contiguous (contig_stride > 0, uniform_len).
 int run_decode(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, int64_t contig_stride,
                int uniform_len, void* out, void* workspace, size_t workspace_bytes, int batch, int q_len, int heads,
                int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale,
-               float softcap, int causal, int num_split, int kernel, void* hip_stream) {
+               float softcap, int causal, int num_split, int kernel, void* hip_stream, const Extras& ex = Extras()) {
   const bool skip_combine = (kernel & MI355_KERNEL_FLAG_SKIP_COMBINE) != 0;
   kernel &= ~MI355_KERNEL_FLAG_SKIP_COMBINE;
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
@@ -126,6 +136,12 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
   p.bt_row_stride = bt_row_stride;
   p.contig_stride = contig_stride;
   p.uniform_len = uniform_len;
+  p.cu_q = ex.cu_q;
+  p.len_excludes_new = ex.len_excludes_new;
+  p.kv_starts = ex.kv_starts;
+  p.scale_per_tensor = ex.scale_per_tensor;
+  p.final_o = ex.final_o;
+  p.final_lse = ex.final_lse;
   p.out = out;
   p.part_o = (float*)workspace;
   p.part_lse = (float*)((char*)workspace + plan.part_o_bytes);
@@ -235,6 +251,114 @@ int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k
                     real_seqlen_kv, out, workspace, workspace_bytes, batch, q_len, heads, heads_kv, dim, kContigTile,
                     (int64_t)batch * kv_seq_stride, q_dtype, kv_dtype, sm_scale, softcap, causal, num_split, kernel,
                     hip_stream);
+}
+
+// Prefill chunk: the workspace holds the decode workspace (shared by the two runs of the fp8 path) and, for an
+// fp8 cache, two sets of fp32 rows + LSE.
+static size_t prefill_final_bytes(int64_t total_q, int heads, int dim) {
+  return align256((size_t)total_q * heads * dim * sizeof(float)) + align256((size_t)total_q * heads * sizeof(float));
+}
+
+static int prefill_plans(int batch, int max_seqlen_q, int heads, int heads_kv, int dim, int page_size,
+                         int64_t max_pages_per_req, int q_dtype, int cache_dtype, int kernel, Plan* cache_plan, Plan* chunk_plan) {
+  int rc = make_plan(batch, max_seqlen_q, heads, heads_kv, dim, page_size, max_pages_per_req, q_dtype, cache_dtype, 0.f, 0,
+                     kernel, cache_plan);
+  if (rc) return rc;
+  *chunk_plan = Plan();
+  if (cache_dtype == MI355_DT_FP8_E4M3FN)  // the chunk's own 16-bit tokens are a second, contiguous key set
+    rc = make_plan(batch, max_seqlen_q, heads, heads_kv, dim, kContigTile, ((int64_t)max_seqlen_q + kContigTile - 1) / kContigTile,
+                   q_dtype, q_dtype, 0.f, 0, kernel, chunk_plan);
+  return rc;
+}
+
+int mi355_gqa_prefill_paged_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
+                                      int page_size, int64_t max_pages_per_req, int q_dtype, int cache_dtype, int kernel,
+                                      size_t* workspace_bytes) {
+  int rc = check_shape(batch, max_seqlen_q, heads, heads_kv, dim, page_size, q_dtype, cache_dtype);
+  if (rc) return rc;
+  if (total_q < 0) return fail(MI355_EINVAL, "total_q must be non-negative");
+  Plan a, b;
+  rc = prefill_plans(batch, max_seqlen_q, heads, heads_kv, dim, page_size, max_pages_per_req, q_dtype, cache_dtype, kernel, &a, &b);
+  if (rc) return rc;
+  size_t wa = a.part_o_bytes + a.part_lse_bytes, wb = b.part_o_bytes + b.part_lse_bytes;
+  size_t total = wa > wb ? wa : wb;
+  if (cache_dtype == MI355_DT_FP8_E4M3FN) total += 2 * prefill_final_bytes(total_q, heads, dim);
+  if (workspace_bytes) *workspace_bytes = total;
+  return MI355_OK;
+}
+
+int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new, void* k_pages, void* v_pages,
+                            const float* k_scale, const float* v_scale, const int32_t* cu_seqlens_q,
+                            const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,
+                            void* workspace, size_t workspace_bytes, int batch, int max_seqlen_q, int64_t total_q, int heads,
+                            int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype, int cache_dtype,
+                            float sm_scale, float softcap, int causal, int kernel, void* hip_stream) {
+  int rc = check_shape(batch, max_seqlen_q, heads, heads_kv, dim, page_size, q_dtype, cache_dtype);
+  if (rc) return rc;
+  if (batch == 0 || total_q == 0) return MI355_OK;
+  if (total_q < 0) return fail(MI355_EINVAL, "total_q must be non-negative");
+  if (!q || !k_new || !v_new || !k_pages || !v_pages || !cu_seqlens_q || !cache_seqlens || !block_table || !out)
+    return fail(MI355_EINVAL, "q, k_new, v_new, k_pages, v_pages, cu_seqlens_q, cache_seqlens, block_table and out must be non-null");
+  const bool fp8 = cache_dtype == MI355_DT_FP8_E4M3FN;
+  if (fp8 && (!k_scale || !v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale are required with an fp8 KV cache");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens, page_size);
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (((uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15)
+    return fail(MI355_EINVAL, "k_new, v_new, k_pages and v_pages must be 16-byte aligned");
+  size_t need = 0;
+  rc = mi355_gqa_prefill_paged_workspace(batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype,
+                                         cache_dtype, kernel, &need);
+  if (rc) return rc;
+  if (need > 0) {
+    if (!workspace) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got null", need);
+    if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
+  }
+  hipStream_t s = (hipStream_t)hip_stream;
+  const char* err = launch_kv_append_chunk(k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens,
+                                           block_table, bt_row_stride, batch, total_q, heads_kv, dim, page_size,
+                                           n_phys_tokens / page_size, q_dtype, cache_dtype, s);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  Extras ex;
+  ex.cu_q = cu_seqlens_q;
+  if (!fp8) {
+    // 16-bit cache: the chunk is in the pages now, bit for bit; one pass over (old + new) tokens
+    ex.len_excludes_new = 1;
+    return run_decode(q, k_pages, v_pages, nullptr, nullptr, cache_seqlens, block_table, bt_row_stride, 0, 0, out, workspace,
+                      workspace_bytes, batch, max_seqlen_q, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype,
+                      cache_dtype, sm_scale, softcap, causal, 0, kernel, hip_stream, ex);
+  }
+  // fp8 cache: the old tokens come dequantised from the pages (every query sees all of them), the chunk's own tokens
+  // unquantised from k_new / v_new (causal inside the chunk) -- gqa_fwd.py:1180-1245 -- and the two results are merged.
+  const size_t fin = prefill_final_bytes(total_q, heads, dim);
+  const size_t o_bytes = align256((size_t)total_q * heads * dim * sizeof(float));
+  char* tail = (char*)workspace + (need - 2 * fin);
+  float* o_a = (float*)tail;
+  float* lse_a = (float*)(tail + o_bytes);
+  float* o_b = (float*)(tail + fin);
+  float* lse_b = (float*)(tail + fin + o_bytes);
+  ex.scale_per_tensor = 1;
+  ex.final_o = o_a;
+  ex.final_lse = lse_a;
+  rc = run_decode(q, k_pages, v_pages, k_scale, v_scale, cache_seqlens, block_table, bt_row_stride, 0, 0, out, workspace,
+                  need - 2 * fin, batch, max_seqlen_q, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype, cache_dtype,
+                  sm_scale, softcap, 0, 0, kernel, hip_stream, ex);
+  if (rc) return rc;
+  Extras eb;
+  eb.cu_q = cu_seqlens_q;
+  eb.len_excludes_new = 1;  // with no seqlens array: length = the chunk's own length
+  eb.kv_starts = cu_seqlens_q;
+  eb.final_o = o_b;
+  eb.final_lse = lse_b;
+  rc = run_decode(q, k_new, v_new, nullptr, nullptr, nullptr, nullptr, ((int64_t)max_seqlen_q + kContigTile - 1) / kContigTile, 0, 0,
+                  out, workspace, need - 2 * fin, batch, max_seqlen_q, heads, heads_kv, dim, kContigTile,
+                  ((total_q + kContigTile - 1) / kContigTile) * kContigTile, q_dtype, q_dtype, sm_scale, softcap, causal, 0, kernel,
+                  hip_stream, eb);
+  if (rc) return rc;
+  err = launch_merge_two(o_a, lse_a, o_b, lse_b, out, total_q * heads, dim, q_dtype, s);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  return MI355_OK;
 }
 
 int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,

@@ -26,6 +26,17 @@ struct DecodeParams {
   // [b*contig_stride, b*contig_stride + uniform_len) of k/v, and page_size is only the tile granule.
   int64_t contig_stride;
   int uniform_len;
+  // Packed variable-length queries (prefill chunks): q and out are [total_q, heads, dim], sequence b owns query rows
+  // [cu_q[b], cu_q[b+1]); q_len is then the largest chunk.  Null = every sequence has q_len query tokens.
+  const int32_t* cu_q;
+  int len_excludes_new;  // with cu_q: seqlens[b] counts the context *before* the chunk; the chunk's tokens are added
+  // Packed contiguous keys/values (the chunk's own tokens): sequence b occupies tokens [kv_starts[b], ...) of k/v.
+  const int32_t* kv_starts;
+  int scale_per_tensor;  // fp8: k_scale/v_scale hold one value each instead of one per (token, kv head)
+  // When set, the result leaves as fp32 rows plus log2-domain log-sum-exp ([total_q, heads, dim] / [total_q, heads])
+  // instead of 16-bit rows in out, so that two calls over disjoint key sets can be merged afterwards.
+  float* final_o;
+  float* final_lse;
   void* out;
   float* part_o;    // workspace: normalised partial outputs, fp32
   float* part_lse;  // workspace: log2-domain log-sum-exp per partial (-inf = empty)
@@ -47,7 +58,17 @@ struct DecodeParams {
 };
 
 // Context length of sequence b: per-sequence array (paged cache) or one value for all (contiguous cache).
-__device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) { return p.seqlens ? p.seqlens[b] : p.uniform_len; }
+__device__ __forceinline__ int q_len_of(const DecodeParams& p, int b) { return p.cu_q ? p.cu_q[b + 1] - p.cu_q[b] : p.q_len; }
+__device__ __forceinline__ int64_t q_row0_of(const DecodeParams& p, int b) { return p.cu_q ? (int64_t)p.cu_q[b] : (int64_t)b * p.q_len; }
+__device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) {
+  int len = p.seqlens ? p.seqlens[b] : p.uniform_len;
+  if (p.cu_q) {
+    const int ql = p.cu_q[b + 1] - p.cu_q[b];
+    if (ql <= 0) return 0;  // no query rows: nothing to compute, the sequence contributes no tile
+    if (p.len_excludes_new) len += ql;
+  }
+  return len;
+}
 
 // Number of KV splits of one sequence and the (tile-aligned) tokens per split, generic kernel.
 // Used identically by the attention kernel and its combine kernel.
@@ -72,6 +93,12 @@ const char* launch_mfma(const DecodeParams& p, int q_dtype, int kv_dtype, bool s
 const char* launch_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
                                 void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size,
                                 int64_t n_pages, hipStream_t s);
+const char* launch_kv_append_chunk(const void* k_new, const void* v_new, void* k_pages, void* v_pages, const float* k_scale,
+                                   const float* v_scale, const int32_t* cu_q, const int32_t* cache_seqlens,
+                                   const int32_t* block_table, int64_t bt_row_stride, int batch, int64_t total_q, int heads_kv,
+                                   int dim, int page_size, int64_t n_pages, int x_dtype, int cache_dtype, hipStream_t s);
+const char* launch_merge_two(const float* o_a, const float* lse_a, const float* o_b, const float* lse_b, void* out,
+                             int64_t rows, int dim, int q_dtype, hipStream_t s);
 const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, const int32_t* seqlens,
                                  const int32_t* block_table, int64_t bt_row_stride, int batch, int heads_kv, int dim,
                                  int page_size, int64_t n_pages, int x_dtype, hipStream_t s);

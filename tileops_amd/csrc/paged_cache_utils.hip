@@ -89,4 +89,107 @@ const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, c
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
+// Append a packed chunk of new tokens to the paged cache: token t of sequence b (t in [cu_q[b], cu_q[b+1])) goes to
+// logical position cache_seqlens[b] + (t - cu_q[b]).  16-bit cache: the row is copied.  FP8 cache: per-tensor scale,
+// q = e4m3fn(clamp(x / scale, -448, 448)) -- the append of the reference's paged prefill kernels
+// (src/tileops/kernels/attention/gqa_fwd.py:1059-1061, :1124-1168).  One workgroup per token, K and V together.
+template <typename XT, bool FP8C>
+__global__ __launch_bounds__(256) void kv_append_chunk_kernel(const uint16_t* __restrict__ k_new, const uint16_t* __restrict__ v_new,
+                                                              void* __restrict__ k_pages, void* __restrict__ v_pages,
+                                                              const float* __restrict__ k_scale, const float* __restrict__ v_scale,
+                                                              const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
+                                                              const int32_t* __restrict__ block_table, int64_t bt_row_stride,
+                                                              int batch, int64_t row_elems, int page_size, int64_t n_pages) {
+  const int64_t t = blockIdx.x;
+  int lo = 0, hi = batch;  // the sequence with cu_q[b] <= t < cu_q[b+1] (empty chunks are skipped by the search)
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int b = lo;
+  if (t >= cu_q[b + 1]) return;
+  const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
+  const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages);
+  const uint16_t* ks = k_new + t * row_elems;
+  const uint16_t* vs = v_new + t * row_elems;
+  if (!FP8C) {
+    uint16_t* kd = (uint16_t*)k_pages + phys * row_elems;
+    uint16_t* vd = (uint16_t*)v_pages + phys * row_elems;
+    for (int64_t i = threadIdx.x * 2; i < row_elems; i += 512) {  // head dims are even: two elements per access
+      *(uint32_t*)(kd + i) = *(const uint32_t*)(ks + i);
+      *(uint32_t*)(vd + i) = *(const uint32_t*)(vs + i);
+    }
+  } else {
+    const float sk = k_scale[0], sv = v_scale[0];
+    uint8_t* kd = (uint8_t*)k_pages + phys * row_elems;
+    uint8_t* vd = (uint8_t*)v_pages + phys * row_elems;
+    for (int64_t i = threadIdx.x * 2; i < row_elems; i += 512) {
+      uint32_t kraw[1] = {*(const uint32_t*)(ks + i)}, vraw[1] = {*(const uint32_t*)(vs + i)};
+      float kf[2], vf[2];
+      Unpack<XT, 2>::run(kraw, kf);
+      Unpack<XT, 2>::run(vraw, vf);
+      const float k0 = fminf(fmaxf(kf[0] / sk, -448.0f), 448.0f), k1 = fminf(fmaxf(kf[1] / sk, -448.0f), 448.0f);
+      const float v0 = fminf(fmaxf(vf[0] / sv, -448.0f), 448.0f), v1 = fminf(fmaxf(vf[1] / sv, -448.0f), 448.0f);
+      *(uint16_t*)(kd + i) = (uint16_t)(__builtin_amdgcn_cvt_pk_fp8_f32(k0, k1, 0u, false) & 0xffff);
+      *(uint16_t*)(vd + i) = (uint16_t)(__builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, 0u, false) & 0xffff);
+    }
+  }
+}
+
+const char* launch_kv_append_chunk(const void* k_new, const void* v_new, void* k_pages, void* v_pages, const float* k_scale,
+                                   const float* v_scale, const int32_t* cu_q, const int32_t* cache_seqlens,
+                                   const int32_t* block_table, int64_t bt_row_stride, int batch, int64_t total_q, int heads_kv,
+                                   int dim, int page_size, int64_t n_pages, int x_dtype, int cache_dtype, hipStream_t s) {
+  if (batch == 0 || total_q == 0) return nullptr;
+  const int64_t row_elems = (int64_t)heads_kv * dim;
+  const bool fp8 = cache_dtype == MI355_DT_FP8_E4M3FN, bf = x_dtype == MI355_DT_BF16;
+#define MI355_LAUNCH_APPEND(XT, F8)                                                                                           \
+  hipLaunchKernelGGL((kv_append_chunk_kernel<XT, F8>), dim3((unsigned)total_q), dim3(256), 0, s, (const uint16_t*)k_new,     \
+                     (const uint16_t*)v_new, k_pages, v_pages, k_scale, v_scale, cu_q, cache_seqlens, block_table,           \
+                     bt_row_stride, batch, row_elems, page_size, n_pages)
+  if (fp8 && bf) MI355_LAUNCH_APPEND(bf16_tag, true);
+  else if (fp8) MI355_LAUNCH_APPEND(fp16_tag, true);
+  else if (bf) MI355_LAUNCH_APPEND(bf16_tag, false);
+  else MI355_LAUNCH_APPEND(fp16_tag, false);
+#undef MI355_LAUNCH_APPEND
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
+// Merge two attention results over disjoint key sets, given as fp32 rows with log2-domain log-sum-exp:
+//   out = (2^(lse_a - m) * o_a + 2^(lse_b - m) * o_b) / (2^(lse_a - m) + 2^(lse_b - m)),  m = max(lse_a, lse_b);
+// a row both sides left empty (-inf, -inf) becomes zero.  One thread per two head elements.
+template <typename QT>
+__global__ __launch_bounds__(256) void merge_two_kernel(const float* __restrict__ o_a, const float* __restrict__ lse_a,
+                                                        const float* __restrict__ o_b, const float* __restrict__ lse_b,
+                                                        uint32_t* __restrict__ out, int64_t rows, int half_dim) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * half_dim) return;
+  const int64_t row = idx / half_dim;
+  const float la = lse_a[row], lb = lse_b[row], m = fmaxf(la, lb);
+  float r0 = 0.f, r1 = 0.f;
+  if (m > -INFINITY) {
+    const float wa = exp2f(la - m), wb = exp2f(lb - m), inv = 1.0f / (wa + wb);
+    const f32x2 a = *(const f32x2*)(o_a + 2 * idx), b = *(const f32x2*)(o_b + 2 * idx);
+    r0 = (wa != 0.f ? wa * a[0] : 0.f) + (wb != 0.f ? wb * b[0] : 0.f);
+    r1 = (wa != 0.f ? wa * a[1] : 0.f) + (wb != 0.f ? wb * b[1] : 0.f);
+    r0 *= inv;
+    r1 *= inv;
+  }
+  out[idx] = (uint32_t)f32_to_elem_bits<QT>(r0) | ((uint32_t)f32_to_elem_bits<QT>(r1) << 16);
+}
+
+const char* launch_merge_two(const float* o_a, const float* lse_a, const float* o_b, const float* lse_b, void* out,
+                             int64_t rows, int dim, int q_dtype, hipStream_t s) {
+  if (rows == 0) return nullptr;
+  const int64_t n = rows * (dim / 2);
+  const unsigned grid = (unsigned)((n + 255) / 256);
+  if (q_dtype == MI355_DT_BF16)
+    hipLaunchKernelGGL(merge_two_kernel<bf16_tag>, dim3(grid), dim3(256), 0, s, o_a, lse_a, o_b, lse_b, (uint32_t*)out, rows, dim / 2);
+  else
+    hipLaunchKernelGGL(merge_two_kernel<fp16_tag>, dim3(grid), dim3(256), 0, s, o_a, lse_a, o_b, lse_b, (uint32_t*)out, rows, dim / 2);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
 }  // namespace mi355

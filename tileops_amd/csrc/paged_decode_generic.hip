@@ -54,19 +54,20 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
   const int t_end = min(len, t_begin + chunk);
   const int32_t* bt_row = p.block_table + (int64_t)b * p.bt_row_stride;
 
+  const int q_len_b = q_len_of(p, b), rows_b = q_len_b * p.group;
+  const int64_t q_row0 = q_row0_of(p, b);
   float qf[RB][EPL];
   int limit[RB];
 #pragma unroll
   for (int rr = 0; rr < RB; rr++) {
     int r = r0 + rr;
-    bool valid = r < p.rows;
+    bool valid = r < rows_b;
     int s = valid ? r / p.group : 0, gidx = valid ? r % p.group : 0;
-    const char* qp = (const char*)p.q +
-                     ((((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gidx) * D + c * EPL) * QB;
+    const char* qp = (const char*)p.q + (((q_row0 + s) * p.heads + kvh * p.group + gidx) * D + c * EPL) * QB;
     uint32_t raw[EPL * QB / 4];
     load_raw<EPL * QB>(qp, raw);
     Unpack<QT, EPL>::run(raw, qf[rr]);
-    limit[rr] = valid ? ((p.causal && p.q_len > 1) ? len - p.q_len + s + 1 : len) : 0;
+    limit[rr] = valid ? ((p.causal && p.q_len > 1) ? len - q_len_b + s + 1 : len) : 0;
   }
 
   float m[RB], l[RB], acc[RB][EPL];
@@ -79,15 +80,15 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
   }
 
   for (int t = t_begin + gi; t < t_end; t += 16) {
-    const int64_t phys = p.contig_stride ? (int64_t)b * p.contig_stride + t : physical_token(bt_row, t, p.page_size, p.n_pages);
+    const int64_t phys = p.kv_starts ? (int64_t)p.kv_starts[b] + t : p.contig_stride ? (int64_t)b * p.contig_stride + t : physical_token(bt_row, t, p.page_size, p.n_pages);
     const int64_t row = phys * p.heads_kv + kvh;
     uint32_t kraw[EPL * KB / 4], vraw[EPL * KB / 4];
     load_raw<EPL * KB>((const char*)p.k + (row * D + c * EPL) * KB, kraw);
     load_raw<EPL * KB>((const char*)p.v + (row * D + c * EPL) * KB, vraw);
     float ks = 1.f, vs = 1.f;
     if (FP8) {
-      ks = p.k_scale[row];
-      vs = p.v_scale[row];
+      ks = p.k_scale[p.scale_per_tensor ? 0 : row];
+      vs = p.v_scale[p.scale_per_tensor ? 0 : row];
     }
     float kf[EPL], vf[EPL];
     Unpack<KVT, EPL>::run(kraw, kf);
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
   for (int idx = tid; idx < RB * D; idx += 256) {
     int rr = idx / D, d = idx - rr * D;
     int r = r0 + rr;
-    if (r >= p.rows) continue;
+    if (r >= rows_b) continue;
     float M = fmaxf(fmaxf(sm_m[0][rr], sm_m[1][rr]), fmaxf(sm_m[2][rr], sm_m[3][rr]));
     float L = 0.f, A = 0.f;
 #pragma unroll
@@ -165,8 +166,13 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
     float o = L > 0.f ? A / L : 0.f;
     int s = r / p.group, gidx = r % p.group;
     if (direct) {
-      uint16_t* op = (uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gidx) * D + d;
-      *op = f32_to_elem_bits<QT>(o);
+      const int64_t orow = (q_row0 + s) * p.heads + kvh * p.group + gidx;
+      if (p.final_o) {
+        p.final_o[orow * D + d] = o;
+        if (d == 0) p.final_lse[orow] = L > 0.f ? M + log2f(L) : -INFINITY;
+      } else {
+        *((uint16_t*)p.out + orow * D + d) = f32_to_elem_bits<QT>(o);
+      }
     } else {
       // partial slot (b, split); rows of all kv heads side by side: global row = kvh*rows + r
       int64_t slot = (int64_t)b * p.max_splits + split;
@@ -200,9 +206,15 @@ __global__ void paged_decode_generic_combine_kernel(const DecodeParams p) {
   }
   float o = W > 0.f ? A / W : 0.f;
   int kvh = grow_in / p.rows, r = grow_in % p.rows;
+  if (r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
   int s = r / p.group, gidx = r % p.group;
-  uint16_t* op = (uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gidx) * p.dim + d;
-  *op = f32_to_elem_bits<QT>(o);
+  const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gidx;
+  if (p.final_o) {
+    p.final_o[orow * p.dim + d] = o;
+    if (d == 0) p.final_lse[orow] = W > 0.f ? M + log2f(W) : -INFINITY;
+  } else {
+    *((uint16_t*)p.out + orow * p.dim + d) = f32_to_elem_bits<QT>(o);
+  }
 }
 
 template <typename QT, typename KVT, int D, int RB>

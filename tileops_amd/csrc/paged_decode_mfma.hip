@@ -381,6 +381,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       int last_pg = (cu.len - 1) >> 4;
       ptok0 = phys_page(cu, cu.pg) * 16;
       ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
+    } else if (p.kv_starts) {
+      ptok0 = (int64_t)p.kv_starts[cu.b] + tok0;  // packed contiguous keys: sequence b starts at kv_starts[b]
     } else if (p.contig_stride) {
       ptok0 = (int64_t)cu.b * p.contig_stride + tok0;  // contiguous cache: no table, a tile never straddles anything
     } else {
@@ -418,7 +420,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     if (FP8) {
       int tk = min(lane & 31, nvalid - 1);
       int64_t ptok = ps16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
-      const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + ptok * p.heads_kv + kvh;
+      const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + (p.scale_per_tensor ? 0 : ptok * p.heads_kv + kvh);
       dma4(lds + 2 * G::KBYTES, sp);
     }
   };
@@ -432,13 +434,17 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   const bool softcap = p.softcap > 0.f;
   const uint32_t q_sign = p.negate_q ? 0x80008000u : 0u;
 
+  int seg_q_len = p.q_len;   // query tokens of the sequence being processed (varies with packed queries)
+  int64_t seg_q_row0 = 0;    // its first row in q / out
   auto begin_segment = [&](const Cursor& cu) __attribute__((always_inline)) {
+    seg_q_len = uni(q_len_of(p, cu.b));
+    seg_q_row0 = (int64_t)uni((int)q_row0_of(p, cu.b));
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
       int r = rg * (16 * NRB) + rb * 16 + c;
-      bool valid = r < p.rows;
+      bool valid = r < seg_q_len * p.group;
       int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
-      const char* qp = (const char*)p.q + ((((int64_t)cu.b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) * 2;
+      const char* qp = (const char*)p.q + (((seg_q_row0 + s) * p.heads + kvh * p.group + gi) * kD) * 2;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         // head elements this lane contributes to k-step j: 8 consecutive ones, matching the K operand
@@ -446,7 +452,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
         u32x4 z = {0, 0, 0, 0};
         qreg[rb][j] = valid ? *(const u32x4*)(qp + d0 * 2) : z;
       }
-      limit[rb] = valid ? ((p.causal && p.q_len > 1) ? cu.len - p.q_len + s + 1 : cu.len) : 0;
+      limit[rb] = valid ? ((p.causal && p.q_len > 1) ? cu.len - seg_q_len + s + 1 : cu.len) : 0;
       m_run[rb] = kNegFloor;
       l_run[rb] = 0.f;
 #pragma unroll
@@ -637,10 +643,17 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       int r = rg * (16 * NRB) + rb * 16 + c;
       float l_tot = group_sum(l_run[rb]);
       float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-      if (r >= p.rows) continue;
+      if (r >= seg_q_len * p.group) continue;
       if (complete) {
         int s = r / p.group, gi = r - s * p.group;
-        uint16_t* op = (uint16_t*)p.out + (((int64_t)cu.b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD;
+        const int64_t orow = (seg_q_row0 + s) * p.heads + kvh * p.group + gi;
+        if (p.final_o) {  // fp32 rows + LSE for a later merge with another call
+#pragma unroll
+          for (int db = 0; db < 8; db++) *(f32x4*)(p.final_o + orow * kD + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+          if (g == 0) p.final_lse[orow] = l_tot > 0.f ? m_run[rb] + log2f(l_tot) : -INFINITY;
+          continue;
+        }
+        uint16_t* op = (uint16_t*)p.out + orow * kD;
 #pragma unroll
         for (int db = 0; db < 8; db++) {
           f32x4 o = o_acc[rb][db] * inv;
@@ -778,11 +791,21 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
   const int b = blockIdx.y, row_all = blockIdx.x, lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
   const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
   const int s = r / p.group, gi = r - s * p.group;
-  uint32_t* op = (uint32_t*)((uint16_t*)p.out + (((int64_t)b * p.q_len + s) * p.heads + kvh * p.group + gi) * kD) + lane;
+  if (p.cu_q && r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
+  const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
+  uint32_t* op = (uint32_t*)((uint16_t*)p.out + orow * kD) + lane;
+  auto store = [&](float a0, float a1, float lse) {
+    if (p.final_o) {
+      *(f32x2*)(p.final_o + orow * kD + 2 * lane) = f32x2{a0, a1};
+      if (lane == 0) p.final_lse[orow] = lse;
+    } else {
+      *op = Mma<QT>::pack(a0, a1);
+    }
+  };
   const int4 rec = ((const int4*)ws_prefix)[b];  // the only load everything else depends on
   const int p_first = rec.y, p_last = rec.z;
   if (p_first < 0) {  // empty sequence: the attention kernel never visits it
-    if (wave == 0) *op = 0;
+    if (wave == 0) store(0.f, 0.f, -INFINITY);
     return;
   }
   if (p_first == p_last) return;  // one wave covered the whole sequence and wrote the output itself
@@ -856,7 +879,7 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
     }
   }
   const float inv = W > 0.f ? 1.0f / W : 0.f;
-  *op = Mma<QT>::pack(acc0 * inv, acc1 * inv);
+  store(acc0 * inv, acc1 * inv, W > 0.f ? M + log2f(W) : -INFINITY);
 }
 
 // Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an

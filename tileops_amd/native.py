@@ -29,6 +29,8 @@ EXPORTED_SYMBOLS = (
     "mi355_gqa_paged_decode",
     "mi355_gqa_decode_workspace",
     "mi355_gqa_decode",
+    "mi355_gqa_prefill_paged_workspace",
+    "mi355_gqa_prefill_paged",
     "mi355_gather_probe",
     "mi355_kv_append_fp8",
 )
@@ -70,6 +72,16 @@ def _declare(lib: ctypes.CDLL) -> None:
         _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_sz,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int,
         _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
+    ]
+    lib.mi355_gqa_prefill_paged_workspace.restype = _c_int
+    lib.mi355_gqa_prefill_paged_workspace.argtypes = [
+        _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, ctypes.POINTER(_c_sz),
+    ]
+    lib.mi355_gqa_prefill_paged.restype = _c_int
+    lib.mi355_gqa_prefill_paged.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
+        _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
+        _c_f32, _c_f32, _c_int, _c_int, _c_vp,
     ]
     lib.mi355_gather_probe.restype = _c_int
     lib.mi355_gather_probe.argtypes = [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_int, _c_i64, _c_i64, _c_int, _c_i64, _c_vp]
@@ -209,6 +221,34 @@ def contiguous_decode(
         batch, q_len, heads, heads_kv, dim, k.shape[1], int(real_seqlen_kv),
         dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
         int(num_split), int(kernel), _stream_ptr(q.device)))
+
+
+def prefill_paged_workspace(batch: int, max_seqlen_q: int, total_q: int, heads: int, heads_kv: int, dim: int, page_size: int,
+                            max_pages_per_req: int, q_dtype: torch.dtype, cache_dtype: torch.dtype,
+                            kernel: int = KERNEL_AUTO) -> int:
+    """Workspace bytes of a paged prefill call.  Touches no device."""
+    lib = load()
+    nbytes = _c_sz(0)
+    _check(lib.mi355_gqa_prefill_paged_workspace(
+        batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, max_pages_per_req, dtype_code(q_dtype),
+        dtype_code(cache_dtype), kernel, ctypes.byref(nbytes)))
+    return int(nbytes.value)
+
+
+def prefill_paged(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                  k_scale: torch.Tensor, v_scale: torch.Tensor, cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor,
+                  block_table: torch.Tensor, out: torch.Tensor, workspace: Optional[torch.Tensor], *, batch: int,
+                  max_seqlen_q: int, heads: int, heads_kv: int, dim: int, page_size: int, sm_scale: float, softcap: float,
+                  causal: bool, kernel: int = KERNEL_AUTO) -> None:
+    """Enqueue one paged prefill call (append + attention) on the current stream of ``q.device``."""
+    lib = load()
+    _check(lib.mi355_gqa_prefill_paged(
+        q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), k_scale.data_ptr(),
+        v_scale.data_ptr(), cu_seqlens_q.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        out.data_ptr(), workspace.data_ptr() if workspace is not None else None,
+        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, k_pages.shape[0], dtype_code(q.dtype),
+        dtype_code(k_pages.dtype), float(sm_scale), float(softcap), int(bool(causal)), int(kernel), _stream_ptr(q.device)))
 
 
 def gather_probe(cache: torch.Tensor, seqlens: torch.Tensor, block_table: torch.Tensor, page_size: int, max_len: int) -> torch.Tensor:
