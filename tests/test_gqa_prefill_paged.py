@@ -1,0 +1,242 @@
+"""Paged prefill chunk with cache append: pins of the CPU oracle (no GPU) and GPU parity through the op layer and the C ABI.
+
+The GPU block restates the reference's test file (tests/ops/attention/test_gqa_prefill_paged.py:120-415): the same
+eight 16-bit cases and six FP8-cache cases (shapes, interleaved block table, scales 0.02, inputs scaled by 0.5), the
+same tolerances (fp16 5e-3/1e-5, bf16 8e-2/1e-2, FP8 cache 8e-2/2e-2), the same three checks -- output, appended rows
+(bit-exact for FP8), untouched old rows -- and the scale validation cases (:418-470).  Fused RoPE (:473-) has no
+counterpart here.  Beyond the reference: head_dim 128 (MFMA kernel), empty chunks and empty caches, both kernels.
+"""
+
+from itertools import accumulate
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle.paged_gqa_decode_ref import (
+    physical_pos, quantize_per_tensor, ref_gqa_prefill_paged, ref_paged_gqa_decode,
+)
+from tests.conftest import require_gfx950
+from tileops_amd import native
+from tileops_amd.ops import GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp as PrefillOp
+from tileops_amd.roofline import gqa_prefill_paged_with_kv_cache_fwd_roofline
+
+DEV = "cuda"
+FP8 = torch.float8_e4m3fn
+TOL = {torch.float16: (5e-3, 1e-5), torch.bfloat16: (8e-2, 1e-2)}
+
+
+def _block_table(batch, max_pages_per_req):
+    """tests/ops/attention/test_gqa_prefill_paged.py:34-40: even pages first, then odd ones."""
+    rows = []
+    for b in range(batch):
+        pages = list(range(b * max_pages_per_req, (b + 1) * max_pages_per_req))
+        rows.append(pages[::2] + pages[1::2])
+    return torch.tensor(rows, dtype=torch.int32)
+
+
+def _case(q_lens, old_lens, heads, heads_kv, dim, dtype, *, fp8=False, page=64, max_pages=8, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    batch, total_q = len(q_lens), sum(q_lens)
+    amp = 0.5 if fp8 else 1.0
+    table = _block_table(batch, max_pages)
+    cu = torch.tensor([0, *accumulate(q_lens)], dtype=torch.int32)
+    cache = torch.tensor(old_lens, dtype=torch.int32)
+    q = torch.randn(total_q, heads, dim, generator=g).to(dtype)
+    k_new = (torch.randn(total_q, heads_kv, dim, generator=g) * amp).to(dtype)
+    v_new = (torch.randn(total_q, heads_kv, dim, generator=g) * amp).to(dtype)
+    scale = torch.tensor([0.02 if fp8 else 1.0])
+    n = batch * max_pages * page
+    k_pages = torch.zeros(n, heads_kv, dim, dtype=FP8 if fp8 else dtype)
+    v_pages = torch.zeros_like(k_pages)
+    for b, old in enumerate(old_lens):  # only the addressed old tokens hold data, as in the reference's fixture
+        ko = (torch.randn(old, heads_kv, dim, generator=g) * amp).to(dtype)
+        vo = (torch.randn(old, heads_kv, dim, generator=g) * amp).to(dtype)
+        for t in range(old):
+            pos = physical_pos(table, b, t, page)
+            k_pages[pos] = quantize_per_tensor(ko[t], scale) if fp8 else ko[t]
+            v_pages[pos] = quantize_per_tensor(vo[t], scale) if fp8 else vo[t]
+    return q, k_new, v_new, k_pages, v_pages, scale, scale.clone(), cu, cache, table
+
+
+# --- oracle pins (CPU) --------------------------------------------------------------------------------------
+def test_oracle_matches_sdpa_with_an_explicit_mask_per_sequence():
+    q_lens, old_lens, H, Hkv, D, page = [5, 12, 1], [20, 0, 70], 8, 2, 32, 16
+    case = _case(q_lens, old_lens, H, Hkv, D, torch.float32, page=page, max_pages=8, seed=3)
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+    for causal in (True, False):
+        out, _, _ = ref_gqa_prefill_paged(*case, page_size=page, is_causal=causal)
+        for b, (n, old) in enumerate(zip(q_lens, old_lens)):
+            q0 = int(cu[b])
+            idx = torch.tensor([physical_pos(table, b, t, page) for t in range(old)], dtype=torch.long)
+            k_all = torch.cat([k_pages[idx], k_new[q0:q0 + n]]).repeat_interleave(H // Hkv, 1).transpose(0, 1)
+            v_all = torch.cat([v_pages[idx], v_new[q0:q0 + n]]).repeat_interleave(H // Hkv, 1).transpose(0, 1)
+            mask = (torch.arange(old + n)[None, :] <= torch.arange(n)[:, None] + old) if causal else None
+            want = F.scaled_dot_product_attention(q[q0:q0 + n].transpose(0, 1), k_all, v_all, attn_mask=mask).transpose(0, 1)
+            torch.testing.assert_close(out[q0:q0 + n], want, atol=2e-5, rtol=1e-5)
+
+
+def test_oracle_row_i_of_a_chunk_is_a_single_token_decode_over_old_tokens_and_the_chunk_up_to_i():
+    """Ties the prefill oracle to the (separately pinned) decode oracle, through the appended pages."""
+    q_lens, old_lens, H, Hkv, D, page = [7, 3], [33, 5], 8, 4, 16, 16
+    case = _case(q_lens, old_lens, H, Hkv, D, torch.float32, page=page, max_pages=8, seed=4)
+    q, _, _, _, _, _, _, cu, cache, table = case
+    out, k_after, v_after = ref_gqa_prefill_paged(*case, page_size=page, is_causal=True, softcap=3.0)
+    for b, (n, old) in enumerate(zip(q_lens, old_lens)):
+        for i in range(n):
+            row = int(cu[b]) + i
+            lens = torch.tensor([old + i + 1], dtype=torch.int32)
+            want = ref_paged_gqa_decode(q[row:row + 1], k_after, v_after, lens, table[b:b + 1], page_size=page, softcap=3.0)
+            torch.testing.assert_close(out[row:row + 1], want, atol=2e-5, rtol=1e-5)
+
+
+def test_oracle_append_touches_exactly_the_chunk_positions_and_quantises_like_a_torch_cast():
+    q_lens, old_lens, page = [9, 0, 4], [60, 17, 0], 32
+    for fp8 in (False, True):
+        case = _case(q_lens, old_lens, 4, 2, 16, torch.float16, fp8=fp8, page=page, max_pages=4, seed=5)
+        _, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+        _, k_after, v_after = ref_gqa_prefill_paged(*case, page_size=page)
+        touched = torch.zeros(k_pages.shape[0], dtype=torch.bool)
+        for b, (n, old) in enumerate(zip(q_lens, old_lens)):
+            for i in range(n):
+                pos = physical_pos(table, b, old + i, page)
+                touched[pos] = True
+                src = k_new[int(cu[b]) + i]
+                want = (src.float() / 0.02).to(FP8) if fp8 else src  # tests/ops/attention/test_gqa_prefill_paged.py:402
+                assert torch.equal(k_after[pos].view(torch.uint8), want.view(torch.uint8))
+        assert touched.sum() == sum(q_lens)
+        assert torch.equal(k_after[~touched].view(torch.uint8), k_pages[~touched].view(torch.uint8))
+        assert torch.equal(v_after[~touched].view(torch.uint8), v_pages[~touched].view(torch.uint8))
+
+
+def test_roofline_formula_by_hand():
+    """src/tileops/perf/formulas.py:567-587 on the reference's llama-8b row: 8 x (512 new, 4096 old), fp16."""
+    flops, nbytes = gqa_prefill_paged_with_kv_cache_fwd_roofline(
+        batch=8, heads=32, heads_kv=8, dim=128, max_pages_per_req=72, page_size=64, max_seqlen_q=512, total_q=4096,
+        q_lens=[512] * 8, cache_lens=[4096] * 8, is_causal=True, dtype="float16")
+    visible = 8 * (512 * 4096 + 512 * 513 // 2)
+    assert flops == 4 * 32 * visible * 128 == 292091330560
+    assert nbytes == (2 * 4096 * 32 * 128 + 2 * 32768 * 8 * 128 + 2 * 2 * 4096 * 8 * 128) * 2 + 9 * 4 + 8 * 4 + 8 * 72 * 4 == 234883396
+    # rows without per-request lengths: deterministic fill (:467-475, :559-565)
+    f2, _ = gqa_prefill_paged_with_kv_cache_fwd_roofline(batch=2, heads=8, heads_kv=2, dim=64, max_pages_per_req=4, page_size=64,
+                                                         max_seqlen_q=100, total_q=150, is_causal=False, dtype="float16")
+    assert f2 == 4 * 8 * (100 * 256 + 50 * 256) * 64
+
+
+def test_op_constructs_without_device_and_validates_like_the_reference():
+    op = PrefillOp(batch=2, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, cache_dtype=FP8, softcap=2.0)
+    assert op.max_cache_len == 512 and op.groups == 4 and op.softcap == 2.0
+    with pytest.raises(ValueError, match="page_size must be a power of two"):
+        PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=48, dim=64)
+    with pytest.raises(ValueError, match="max_position is required when fuse_rope=True"):
+        PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, fuse_rope=True)
+    with pytest.raises(ValueError, match="rotary_dim requires fuse_rope=True"):
+        PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, rotary_dim=32)
+    with pytest.raises(ValueError, match="fuse_rope is not supported with FP8 paged KV cache yet"):
+        PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, fuse_rope=True, max_position=512, cache_dtype=FP8)
+    with pytest.raises(NotImplementedError):
+        _ = op.total_flops
+
+
+# --- GPU parity ---------------------------------------------------------------------------------------------
+def _run(op, case, page, dtype, *, fp8=False, causal=True, softcap=0.0, atol=None, rtol=None):
+    ref, k_after, v_after = ref_gqa_prefill_paged(*case, page_size=page, is_causal=causal, softcap=softcap)
+    dev = [t.to(DEV) for t in case]
+    cu = case[7]
+    q_lens = (cu[1:] - cu[:-1]).tolist()
+    out = op(*dev, max(q_lens))
+    torch.cuda.synchronize()
+    assert isinstance(out, torch.Tensor) and out.shape == case[0].shape and out.dtype == dtype
+    if atol is None:
+        atol, rtol = (8e-2, 2e-2) if fp8 else TOL[dtype]
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=atol, rtol=rtol)
+    # appended rows bit for bit, everything else untouched
+    assert torch.equal(dev[3].cpu().view(torch.uint8), k_after.view(torch.uint8))
+    assert torch.equal(dev[4].cpu().view(torch.uint8), v_after.view(torch.uint8))
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "q_lens, old_lens, heads, heads_kv, dim, is_causal, dtype",
+    [pytest.param([64, 96], [80, 128], 8, 2, 64, True, torch.float16, id="gqa_ratio4_mixed_fp16"),
+     pytest.param([17, 33], [37, 100], 8, 2, 64, True, torch.float16, id="gqa_unaligned_old_len_fp16"),
+     pytest.param([1], [511], 8, 2, 64, True, torch.float16, id="gqa_decode_len_capacity_boundary_fp16"),
+     pytest.param([1, 17], [511, 37], 8, 2, 64, True, torch.float16, id="gqa_mixed_capacity_boundary_fp16"),
+     pytest.param([64, 64], [64, 128], 8, 8, 64, True, torch.float16, id="mha_fp16"),
+     pytest.param([32, 64], [96, 160], 8, 1, 64, True, torch.float16, id="mqa_fp16"),
+     pytest.param([64, 96], [80, 128], 8, 2, 64, False, torch.float16, id="gqa_noncausal_fp16"),
+     pytest.param([64, 96], [80, 128], 8, 2, 64, True, torch.bfloat16, id="gqa_ratio4_bf16")],
+)
+def test_gqa_prefill_paged_with_kv_cache_fwd(q_lens, old_lens, heads, heads_kv, dim, is_causal, dtype):
+    require_gfx950()
+    case = _case(q_lens, old_lens, heads, heads_kv, dim, dtype)
+    op = PrefillOp(batch=len(q_lens), heads=heads, heads_kv=heads_kv, max_pages_per_req=8, page_size=64, dim=dim, is_causal=is_causal)
+    _run(op, case, 64, dtype, causal=is_causal)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "is_causal, softcap, dtype, page_size",
+    [pytest.param(True, None, torch.float16, 64, id="causal-fp16-page64"), pytest.param(False, None, torch.float16, 64, id="noncausal-fp16-page64"),
+     pytest.param(True, 2.0, torch.float16, 64, id="causal-softcap-fp16-page64"), pytest.param(True, None, torch.bfloat16, 64, id="causal-bf16-page64"),
+     pytest.param(True, None, torch.float16, 16, id="causal-fp16-page16"), pytest.param(True, None, torch.float16, 128, id="causal-fp16-page128")],
+)
+def test_gqa_prefill_paged_with_fp8_kv_cache_fwd(is_causal, softcap, dtype, page_size):
+    require_gfx950()
+    case = _case([33, 48], [67, 80], 8, 2, 64, dtype, fp8=True, page=page_size)
+    op = PrefillOp(batch=2, heads=8, heads_kv=2, max_pages_per_req=8, page_size=page_size, dim=64, is_causal=is_causal,
+                   cache_dtype=FP8, softcap=softcap)
+    _run(op, case, page_size, dtype, fp8=True, causal=is_causal, softcap=softcap or 0.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scale_name, bad_value", [("k_scale", 0.0), ("k_scale", -0.01), ("k_scale", float("inf")), ("v_scale", float("nan"))])
+def test_gqa_prefill_paged_with_fp8_kv_cache_rejects_invalid_scales(scale_name, bad_value):
+    require_gfx950()
+    case = [t.to(DEV) for t in _case([1], [0], 8, 2, 64, torch.float16, fp8=True, max_pages=1)]
+    case[5 if scale_name == "k_scale" else 6] = torch.tensor([bad_value], device=DEV)
+    op = PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=1, page_size=64, dim=64, cache_dtype=FP8)
+    with pytest.raises(ValueError, match=f"{scale_name}.*finite positive"):
+        op(*case, 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel", [native.KERNEL_GENERIC, native.KERNEL_AUTO], ids=["general", "mfma"])
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_head_dim_128_empty_chunks_empty_caches_and_both_kernels(kernel, fp8, dtype):
+    """Chunks of 0, 1, 33 and 130 rows (more than one row group per kv head), caches of 0, 5 and 700 tokens, tails that
+    are not tile multiples; the same call on the general kernel and on the MFMA kernel (head_dim 128)."""
+    require_gfx950()
+    q_lens, old_lens = [33, 0, 130, 1, 20], [700, 5, 0, 257, 64]
+    case = _case(q_lens, old_lens, 16, 4, 128, dtype, fp8=fp8, page=32, max_pages=32, seed=11)
+    op = PrefillOp(batch=len(q_lens), heads=16, heads_kv=4, max_pages_per_req=32, page_size=32, dim=128, cache_dtype=FP8 if fp8 else None)
+    call = op.attention_call(dtype, torch.device(DEV, 0))
+    key = op.select_kernel_key(tuple(op.kernel_map), call)
+    assert key == ("gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel" if fp8 else "gqa_prefill_paged_with_kv_cache_fwd_kernel")
+    inputs = [t.to(DEV) for t in case]
+    op._get_kernel(tuple(inputs), key, call).config["kernel"] = kernel
+    tol = (8e-2, 2e-2) if fp8 else ((2e-2, 2e-2) if dtype == torch.bfloat16 else (5e-3, 1e-3))
+    _run(op, case, 32, dtype, fp8=fp8, atol=tol[0], rtol=tol[1])
+
+
+@pytest.mark.gpu
+def test_prefill_rejects_bad_calls():
+    require_gfx950()
+    case = [t.to(DEV) for t in _case([4, 4], [10, 10], 8, 2, 64, torch.float16)]
+    op = PrefillOp(batch=2, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64)
+    with pytest.raises(ValueError, match="max_seqlen_q .3. must be >= actual max Q sequence length .4."):
+        op(*case, 3)
+    bad = list(case)
+    bad[8] = torch.tensor([510, 10], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="exceeds paged KV capacity"):
+        op(*bad, 4)
+    bad = list(case)
+    bad[9] = case[9] + 100
+    with pytest.raises(ValueError, match="block_table references page"):
+        op(*bad, 4)
+    bad = list(case)
+    bad[3] = case[3].to(torch.bfloat16)
+    with pytest.raises(ValueError, match="Expected k_pages.dtype"):
+        op(*bad, 4)

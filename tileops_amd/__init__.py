@@ -1,6 +1,6 @@
 """MI355X (gfx950) paged GQA decode attention behind the TileOPs operator contract.
 
-Public surface: the three ops, the backend seam, the manifest loader.  The HIP library is opened lazily on
+Public surface: the four ops, the backend seam, the manifest loader.  The HIP library is opened lazily on
 the first kernel build; importing this package touches no device.
 """
 
@@ -12,11 +12,13 @@ from .ops import (  # noqa: F401
     GroupedQueryAttentionDecodeWithKVCacheFwdOp,
     GroupedQueryAttentionDecodePagedWithKVCacheFwdOp,
     GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp,
+    GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp,
 )
 
 __all__ = [
     "GroupedQueryAttentionDecodeWithKVCacheFwdOp",
     "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp",
     "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp",
+    "GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp",
 ]
 __version__ = "0.1.0"

@@ -25,12 +25,15 @@ from . import native
 
 __all__ = [
     "AttentionCall", "DECODE_KEYS", "GQADecodeKernel", "GQADecodeMfmaKernel", "GQADecodePagedKernel",
-    "GQADecodePagedMfmaKernel", "Kernel", "PAGED_DECODE_KEYS",
+    "GQADecodePagedMfmaKernel", "GQAPrefillPagedWithFP8KVCacheFwdKernel", "GQAPrefillPagedWithKVCacheFwdKernel", "Kernel",
+    "PAGED_DECODE_KEYS", "PAGED_PREFILL_KEYS", "PrefillCall",
     "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch",
 ]
 
 #: Dispatch keys of the paged decode ops, in no particular order (selection never reads the order).
 PAGED_DECODE_KEYS = ("gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel")
+#: Dispatch keys of the paged prefill op (the reference's third key, the fused-RoPE kernel, has no counterpart here).
+PAGED_PREFILL_KEYS = ("gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel", "gqa_prefill_paged_with_kv_cache_fwd_kernel")
 #: Dispatch keys of the contiguous-cache decode op.
 DECODE_KEYS = ("gqa_decode_kernel", "gqa_decode_mfma_kernel")
 
@@ -422,3 +425,98 @@ class GQADecodeMfmaKernel(GQADecodeKernel):
     @property
     def autotune_configs(self) -> list[dict]:
         return [dict(self.default_config)]
+
+
+@dataclass(frozen=True)
+class PrefillCall:
+    """Facts of one paged prefill call that kernel selection filters on
+    (reference: src/tileops/ops/attention/gqa.py:843-861, the fields of ``attention_call``)."""
+
+    dtype: torch.dtype
+    batch: int
+    heads: int
+    heads_kv: int
+    dim: int
+    max_pages_per_req: int
+    page_size: int
+    is_causal: bool
+    sm_scale: float
+    softcap: float
+    cache_dtype: torch.dtype
+    fuse_rope: bool = False
+    max_position: Optional[int] = None
+    rotary_dim: Optional[int] = None
+    tune: bool = False
+    arch: Optional[int] = None
+
+
+class GQAPrefillPagedWithKVCacheFwdKernel(Kernel):
+    """Packed GQA prefill chunk with paged-cache append, cache element type = attention element type.
+
+    Constructor keywords and ``forward`` argument order follow the reference class
+    (src/tileops/kernels/attention/gqa_fwd.py:938-1003 and its base).  One library call appends the chunk to the
+    pages and runs attention over old + new tokens with the decode kernels (every query row of a chunk is a
+    decode query; chunks of different lengths are packed).  Long chunks re-stream the keys once per 32-64 query
+    rows of a kv head: the layout is right for chunked prefill next to decode, not for long prompts.
+    """
+
+    supported_archs = [GFX950_ARCH]
+    general = True
+    _cache_is_fp8 = False
+
+    @classmethod
+    def applies(cls, call: PrefillCall) -> bool:
+        return not call.fuse_rope and call.cache_dtype == call.dtype
+
+    def __init__(self, *, batch: int, heads: int, heads_kv: int, max_pages_per_req: int, page_size: int, dim: int,
+                 is_causal: bool = True, dtype: Any = "float16", sm_scale: Optional[float] = None, softcap: float = 0.0,
+                 max_position: Optional[int] = None, rotary_dim: Optional[int] = None, config: Optional[dict] = None,
+                 tune: bool = False, device_index: Optional[int] = None) -> None:
+        super().__init__(device_index=device_index)
+        self.batch, self.heads, self.heads_kv, self.dim = batch, heads, heads_kv, dim
+        self.max_pages_per_req, self.page_size, self.is_causal = max_pages_per_req, page_size, is_causal
+        self.dtype = _as_torch_dtype(dtype)
+        self.sm_scale = dim ** -0.5 if sm_scale is None else sm_scale
+        self.softcap = softcap
+        self.init_config(config, tune)
+
+    @property
+    def default_config(self) -> dict[str, Any]:
+        return {"kernel": native.KERNEL_AUTO}
+
+    @property
+    def autotune_configs(self) -> list[dict]:
+        return [{"kernel": native.KERNEL_AUTO}, {"kernel": native.KERNEL_GENERIC}]
+
+    def forward(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pages: torch.Tensor,
+                v_pages: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
+                cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor, block_table: torch.Tensor, max_seqlen_q: int,
+                cos_table: Optional[torch.Tensor] = None, sin_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+        native.require_gfx950(q.device)
+        if cos_table is not None or sin_table is not None:
+            raise NotImplementedError("fused RoPE is not served by the MI355X paged prefill kernels")
+        kernel = int(self.config.get("kernel", native.KERNEL_AUTO))
+        nbytes = native.prefill_paged_workspace(self.batch, max_seqlen_q, q.shape[0], self.heads, self.heads_kv, self.dim,
+                                                self.page_size, block_table.shape[1], q.dtype, k_pages.dtype, kernel)
+        out = torch.empty_like(q)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
+        if k_scale is None:  # never read with a 16-bit cache; the entry point wants a pointer all the same
+            k_scale = v_scale = torch.ones(1, dtype=torch.float32, device=q.device)
+        native.prefill_paged(q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table,
+                             out, workspace, batch=self.batch, max_seqlen_q=max_seqlen_q, heads=self.heads,
+                             heads_kv=self.heads_kv, dim=self.dim, page_size=self.page_size, sm_scale=self.sm_scale,
+                             softcap=self.softcap, causal=self.is_causal, kernel=kernel)
+        return out
+
+
+class GQAPrefillPagedWithFP8KVCacheFwdKernel(GQAPrefillPagedWithKVCacheFwdKernel):
+    """The same call against an FP8-e4m3fn cache with per-tensor scales (reference:
+    src/tileops/kernels/attention/gqa_fwd.py:1005-1460): the chunk is quantised into the pages, attention reads the
+    old tokens dequantised and the chunk's own tokens unquantised (two passes merged by log-sum-exp)."""
+
+    general = False
+    _cache_is_fp8 = True
+
+    @classmethod
+    def applies(cls, call: PrefillCall) -> bool:
+        return not call.fuse_rope and call.cache_dtype == torch.float8_e4m3fn

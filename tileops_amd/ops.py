@@ -25,8 +25,9 @@ import torch
 
 from .backend import Target
 from .kernels import (
-    DECODE_KEYS, PAGED_DECODE_KEYS, AttentionCall, GQADecodeKernel, GQADecodeMfmaKernel, GQADecodePagedKernel,
-    GQADecodePagedMfmaKernel, get_arch,
+    DECODE_KEYS, PAGED_DECODE_KEYS, PAGED_PREFILL_KEYS, AttentionCall, GQADecodeKernel, GQADecodeMfmaKernel,
+    GQADecodePagedKernel, GQADecodePagedMfmaKernel, GQAPrefillPagedWithFP8KVCacheFwdKernel,
+    GQAPrefillPagedWithKVCacheFwdKernel, PrefillCall, get_arch,
 )
 from .op_base import _UNRESOLVED, Op
 
@@ -34,6 +35,7 @@ __all__ = [
     "GroupedQueryAttentionDecodeWithKVCacheFwdOp",
     "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp",
     "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp",
+    "GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp",
 ]
 
 FP8 = torch.float8_e4m3fn
@@ -360,3 +362,192 @@ class GroupedQueryAttentionDecodeWithKVCacheFwdOp(Op):
         if k_scale is None:
             return kernel(q, k, v, real_seqlen_kv)
         return kernel(q, k, v, real_seqlen_kv, k_scale, v_scale)
+
+
+def _paged_cache_dtype(cache_dtype: Optional[torch.dtype]) -> Optional[torch.dtype]:
+    """``None`` follows the attention dtype; otherwise fp16, bf16 or float8_e4m3fn (gqa.py:57-63)."""
+    if cache_dtype is None:
+        return None
+    if cache_dtype != FP8:
+        _validate_attention_dtype(cache_dtype)
+    return cache_dtype
+
+
+class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
+    """Packed GQA prefill with paged KV cache append. Layout: THD.
+
+    The current chunk is packed by request. ``cache_seqlens`` stores each request's logical KV length before append.
+    ``block_table`` maps logical page ids to physical pages in ``k_pages`` / ``v_pages``.
+
+    Keeps the reference op's contract (src/tileops/ops/attention/gqa.py:765-1157): constructor arguments, defaults and
+    messages, the eleven ``forward`` arguments in order, the validation of devices, contiguity, shapes, dtypes, scale
+    values, ``cu_seqlens_q`` / ``cache_seqlens`` consistency, capacity and block-table range (:897-1046; like the
+    reference it reads a few device scalars to do so).  ``fuse_rope=True`` is accepted by the constructor's checks as in
+    the reference but no kernel here serves it: such an op raises when called.
+    """
+
+    def __init__(self, batch: int, heads: int, heads_kv: int, max_pages_per_req: int, page_size: int, dim: int,
+                 is_causal: bool = True, cache_dtype: Optional[torch.dtype] = None, sm_scale: Optional[float] = None,
+                 softcap: Optional[float] = None, kernel_map: Optional[Dict[str, type]] = None, tune: bool = False,
+                 fuse_rope: bool = False, rope_base: float = 10000.0, max_position: Optional[int] = None,
+                 rotary_dim: Optional[int] = None, *, target: Target = None) -> None:
+        _validate_gqa_dims(heads, heads_kv, dim)
+        if fuse_rope:
+            rotary_dim = dim if rotary_dim is None else rotary_dim
+            if rotary_dim <= 0 or rotary_dim % 2 != 0 or rotary_dim > dim:
+                raise ValueError("rotary_dim must be a positive even number no larger than dim")
+            if max_position is None:
+                raise ValueError("max_position is required when fuse_rope=True")
+            _validate_positive(max_position=max_position)
+        elif rotary_dim is not None:
+            raise ValueError("rotary_dim requires fuse_rope=True")
+        _validate_positive(batch=batch, max_pages_per_req=max_pages_per_req, page_size=page_size)
+        if page_size & (page_size - 1) != 0:
+            raise ValueError("page_size must be a power of two")
+        cache_dtype = _paged_cache_dtype(cache_dtype)
+        if fuse_rope and cache_dtype == FP8:
+            raise ValueError("fuse_rope is not supported with FP8 paged KV cache yet")
+        self.batch, self.heads, self.heads_kv, self.groups = batch, heads, heads_kv, heads // heads_kv
+        self.max_pages_per_req, self.page_size = max_pages_per_req, page_size
+        self.max_cache_len = max_pages_per_req * page_size
+        self.dim, self.is_causal, self.cache_dtype = dim, is_causal, cache_dtype
+        self.sm_scale = _attention_scale(dim, sm_scale)
+        self.softcap = _score_softcap(softcap)
+        self.fuse_rope, self.rope_base, self.max_position, self.rotary_dim = fuse_rope, rope_base, max_position, rotary_dim
+        self.tune = tune
+        if target is not None:
+            self.target = target
+        self.dispatch_kernel(kernel_map)
+
+    @property
+    def default_kernel_map(self) -> Dict[str, type]:
+        return {
+            "gqa_prefill_paged_with_kv_cache_fwd_kernel": GQAPrefillPagedWithKVCacheFwdKernel,
+            "gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel": GQAPrefillPagedWithFP8KVCacheFwdKernel,
+        }
+
+    def _resolved_cache_dtype(self, dtype: torch.dtype) -> torch.dtype:
+        return dtype if self.cache_dtype is None else self.cache_dtype
+
+    def attention_call(self, dtype: torch.dtype, device: Optional[torch.device] = None) -> PrefillCall:
+        index = device.index if device is not None and device.type == "cuda" else None
+        return PrefillCall(
+            dtype=dtype, batch=self.batch, heads=self.heads, heads_kv=self.heads_kv, dim=self.dim,
+            max_pages_per_req=self.max_pages_per_req, page_size=self.page_size, is_causal=self.is_causal,
+            sm_scale=self.sm_scale, softcap=self.softcap, cache_dtype=self._resolved_cache_dtype(dtype),
+            fuse_rope=self.fuse_rope, max_position=self.max_position, rotary_dim=self.rotary_dim, tune=self.tune,
+            arch=get_arch(index))
+
+    def _get_kernel(self, inputs: "tuple[torch.Tensor | None, ...]", key: str, call: PrefillCall):
+        device = next((t.device for t in inputs if t is not None), None)
+
+        def build():
+            return self.kernel_map[key](
+                batch=call.batch, heads=call.heads, heads_kv=call.heads_kv, max_pages_per_req=call.max_pages_per_req,
+                page_size=call.page_size, dim=call.dim, is_causal=call.is_causal, dtype=call.dtype, sm_scale=call.sm_scale,
+                softcap=call.softcap, max_position=call.max_position, rotary_dim=call.rotary_dim, tune=call.tune,
+                device_index=device.index if device is not None and device.type == "cuda" else None)
+
+        return self.get_or_build_kernel(key, inputs, key=call.dtype, build=build)
+
+    def _validate_forward_inputs(self, q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens,
+                                 block_table, max_seqlen_q) -> None:
+        tensors = {"q": q, "k_new": k_new, "v_new": v_new, "k_pages": k_pages, "v_pages": v_pages, "k_scale": k_scale,
+                   "v_scale": v_scale, "cu_seqlens_q": cu_seqlens_q, "cache_seqlens": cache_seqlens, "block_table": block_table}
+        for name, t in tensors.items():
+            if t.device.type != "cuda":
+                raise ValueError(f"{name} must be on a cuda device, got {t.device}")
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous")
+        q_tail, kv_tail = (self.heads, self.dim), (self.heads_kv, self.dim)
+        if q.ndim != 3 or tuple(q.shape[1:]) != q_tail:
+            raise ValueError(f"q must have shape [total_q, {self.heads}, {self.dim}], got {q.shape}")
+        if k_new.ndim != 3 or tuple(k_new.shape[1:]) != kv_tail:
+            raise ValueError(f"k_new must have shape [total_q, {self.heads_kv}, {self.dim}], got {k_new.shape}")
+        if v_new.shape != k_new.shape:
+            raise ValueError(f"v_new must have the same shape as k_new, got {v_new.shape} and {k_new.shape}")
+        if k_new.shape[0] != q.shape[0]:
+            raise ValueError(f"k_new.shape[0] ({k_new.shape[0]}) must equal q.shape[0] ({q.shape[0]})")
+        if k_pages.ndim != 3 or tuple(k_pages.shape[1:]) != kv_tail:
+            raise ValueError(f"k_pages must have shape [physical_tokens, {self.heads_kv}, {self.dim}], got {k_pages.shape}")
+        if v_pages.shape != k_pages.shape:
+            raise ValueError(f"v_pages must have the same shape as k_pages, got {v_pages.shape} and {k_pages.shape}")
+        if k_pages.shape[0] % self.page_size != 0:
+            raise ValueError("k_pages physical token dimension must be divisible by page_size")
+        if k_scale.shape != (1,) or v_scale.shape != (1,):
+            raise ValueError(f"k_scale and v_scale must have shape (1,), got {k_scale.shape} and {v_scale.shape}")
+        if cu_seqlens_q.shape != (self.batch + 1,):
+            raise ValueError(f"cu_seqlens_q shape must be ({self.batch + 1},), got {tuple(cu_seqlens_q.shape)}")
+        if cache_seqlens.shape != (self.batch,):
+            raise ValueError(f"cache_seqlens shape must be ({self.batch},), got {tuple(cache_seqlens.shape)}")
+        if block_table.shape != (self.batch, self.max_pages_per_req):
+            raise ValueError(f"block_table shape must be ({self.batch}, {self.max_pages_per_req}), got {tuple(block_table.shape)}")
+        _validate_attention_dtype(q.dtype)
+        cache_dtype = self._resolved_cache_dtype(q.dtype)
+        if cache_dtype != q.dtype and cache_dtype != FP8:
+            raise ValueError(f"cache_dtype must be either same as the q element type or torch.float8_e4m3fn, got {cache_dtype}")
+        for name, t in (("k_new", k_new), ("v_new", v_new)):
+            if t.dtype != q.dtype:
+                raise ValueError(f"Expected {name}.dtype {q.dtype}, got {t.dtype}")
+        for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
+            if t.dtype != cache_dtype:
+                raise ValueError(f"Expected {name}.dtype {cache_dtype}, got {t.dtype}")
+        for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            if t.dtype != torch.float32:
+                raise ValueError(f"{name} must have dtype torch.float32, got {t.dtype}")
+            if cache_dtype == FP8 and not torch.all(torch.isfinite(t) & (t > 0)).item():
+                raise ValueError(f"{name} must contain finite positive values")
+        for name, t in (("cu_seqlens_q", cu_seqlens_q), ("cache_seqlens", cache_seqlens), ("block_table", block_table)):
+            if t.dtype != torch.int32:
+                raise ValueError(f"{name} must have dtype torch.int32, got {t.dtype}")
+        cu = cu_seqlens_q.cpu()
+        if int(cu[0]) != 0:
+            raise ValueError("cu_seqlens_q[0] must be 0")
+        q_lens = cu[1:] - cu[:-1]
+        if bool((q_lens < 0).any()):
+            raise ValueError("cu_seqlens_q must be non-decreasing")
+        total_q = int(cu[-1])
+        if total_q != q.shape[0]:
+            raise ValueError(f"cu_seqlens_q[-1] ({total_q}) must equal q.shape[0] ({q.shape[0]})")
+        actual_max_q = int(q_lens.max())
+        if max_seqlen_q < actual_max_q:
+            raise ValueError(f"max_seqlen_q ({max_seqlen_q}) must be >= actual max Q sequence length ({actual_max_q})")
+        cache = cache_seqlens.cpu()
+        if int(cache.min()) < 0:
+            raise ValueError("cache_seqlens must be non-negative")
+        max_total_len = int((cache + q_lens).max())
+        if max_total_len > self.max_cache_len:
+            raise ValueError("cache_seqlens + q_len exceeds paged KV capacity: "
+                             f"max total length {max_total_len}, capacity {self.max_cache_len}")
+        num_pages = k_pages.shape[0] // self.page_size
+        min_page, max_page = int(block_table.min().item()), int(block_table.max().item())
+        if min_page < 0:
+            raise ValueError("block_table must contain non-negative physical page ids")
+        if max_page >= num_pages:
+            raise ValueError(f"block_table references page {max_page}, but only {num_pages} pages exist")
+
+    def _infer_output_shapes(self, q_shape, k_new_shape, v_new_shape, k_pages_shape, v_pages_shape, k_scale_shape,
+                             v_scale_shape, cu_seqlens_q_shape, cache_seqlens_shape, block_table_shape) -> dict[str, tuple[int, ...]]:
+        """Manifest ``shape_rules``: ``o.shape == q.shape``."""
+        return {"o": tuple(q_shape)}
+
+    def forward(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pages: torch.Tensor,
+                v_pages: torch.Tensor, k_scale: torch.Tensor, v_scale: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                cache_seqlens: torch.Tensor, block_table: torch.Tensor, max_seqlen_q: int) -> torch.Tensor:
+        self._validate_forward_inputs(q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens,
+                                      block_table, max_seqlen_q)
+        self.dtype = q.dtype
+        inputs = (q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table)
+        call = self.attention_call(q.dtype, q.device)
+        key = self.select_kernel_key(PAGED_PREFILL_KEYS, call)
+        return self._get_kernel(inputs, key, call)(*inputs, max_seqlen_q)
+
+    @property
+    def total_flops(self) -> int:
+        raise NotImplementedError("total_flops is not defined for paged varlen ops; "
+                                  "compute per-sample from cu_seqlens and cache_seqlens at call time.")
+
+    @property
+    def total_memory(self) -> int:
+        raise NotImplementedError("total_memory is not defined for paged varlen ops; "
+                                  "compute per-sample from cu_seqlens and cache_seqlens at call time.")

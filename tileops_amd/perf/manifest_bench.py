@@ -33,8 +33,9 @@ from .. import native
 from ..manifest import load_manifest
 from ..ops import (
     GroupedQueryAttentionDecodePagedWithKVCacheFwdOp, GroupedQueryAttentionDecodeWithKVCacheFwdOp,
-    GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp,
+    GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp, GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp,
 )
+from ..roofline import _distribute_total, gqa_prefill_paged_with_kv_cache_fwd_roofline
 from ..workloads import FP8, GroupedQueryAttentionDecodePagedWorkload, PagedDecodeConfig, gen_paged_inputs, quantize_kv_per_token
 
 HBM_PEAK_TBS = 8.0
@@ -218,10 +219,52 @@ def _contiguous_case(row: dict, dtype: torch.dtype, device: torch.device):
     return op, args, baseline
 
 
+class _PrefillView:
+    """Gives ``eval_roofline`` of a prefill call the per-request lengths of the workload row."""
+
+    def __init__(self, row: dict, dtype: str) -> None:
+        self.row, self.dtype = dict(row), dtype
+
+    def eval_roofline(self) -> tuple[int, int]:
+        return gqa_prefill_paged_with_kv_cache_fwd_roofline(dtype=self.dtype, **{k: v for k, v in self.row.items() if k not in ("dtypes", "label")})
+
+
+def _prefill_case(row: dict, dtype: torch.dtype, device: torch.device):
+    batch, heads, heads_kv, dim = row["batch"], row["heads"], row["heads_kv"], row["dim"]
+    page, max_pages, max_q = row["page_size"], row["max_pages_per_req"], row["max_seqlen_q"]
+    cache_dtype = _DT[row.get("cache_dtype", str(dtype).removeprefix("torch."))]
+    q_lens = row.get("q_lens") or _distribute_total(row["total_q"], batch, max_q)
+    cache_lens = row.get("cache_lens") or [max(max_pages * page - int(n), 0) for n in q_lens]
+    total_q = sum(q_lens)
+    op = GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(
+        batch=batch, heads=heads, heads_kv=heads_kv, max_pages_per_req=max_pages, page_size=page, dim=dim,
+        is_causal=row.get("is_causal", True), cache_dtype=cache_dtype if cache_dtype == FP8 else None, softcap=row.get("softcap"))
+    fp8 = cache_dtype == FP8
+    amp = 0.5 if fp8 else 1.0
+    q = torch.randn(total_q, heads, dim, device=device, dtype=dtype)
+    k_new = (torch.randn(total_q, heads_kv, dim, device=device) * amp).to(dtype)
+    v_new = (torch.randn(total_q, heads_kv, dim, device=device) * amp).to(dtype)
+    n_phys = row["physical_tokens"]
+    scale = torch.tensor([0.02 if fp8 else 1.0], device=device)
+    pool = torch.randn(2, n_phys, heads_kv, dim, device=device) * amp
+    k_pages = (pool[0] / scale).clamp(-448, 448).to(FP8) if fp8 else pool[0].to(dtype)
+    v_pages = (pool[1] / scale).clamp(-448, 448).to(FP8) if fp8 else pool[1].to(dtype)
+    del pool
+    perm = torch.randperm(n_phys // page, device=device)[:batch * max_pages].to(torch.int32)
+    table = perm.reshape(batch, max_pages).contiguous()
+    cu = torch.tensor([0, *torch.tensor(q_lens).cumsum(0).tolist()], dtype=torch.int32, device=device)
+    cache = torch.tensor(cache_lens, dtype=torch.int32, device=device)
+    args = (q, k_new, v_new, k_pages, v_pages, scale, scale.clone(), cu, cache, table, max(q_lens))
+    view_row = dict(row, q_lens=q_lens, cache_lens=cache_lens, total_q=total_q)
+    op.eval_roofline = _PrefillView(view_row, str(dtype).removeprefix("torch.")).eval_roofline
+    return op, args, None
+
+
 _CASES = {
     "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp": lambda r, d, dev: _paged_case(r, d, dev, False),
     "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp": lambda r, d, dev: _paged_case(r, d, dev, True),
     "GroupedQueryAttentionDecodeWithKVCacheFwdOp": _contiguous_case,
+    "GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp": _prefill_case,
 }
 
 
@@ -249,7 +292,7 @@ def main(argv: Optional[list[str]] = None) -> int:
             for dname in row["dtypes"]:
                 dtype = _DT[dname]
                 kv_elems = 2
-                for s in row["kv_shape"]:
+                for s in row.get("kv_shape") or (row["physical_tokens"], row["heads_kv"], row["dim"]):
                     kv_elems *= s
                 if kv_elems * 2 / 2**30 > args.max_kv_gib:
                     print(f"skip {op_name} {row['label']} {dname}: K+V of {kv_elems * 2 / 2**30:.1f} GiB", flush=True)
@@ -260,8 +303,12 @@ def main(argv: Optional[list[str]] = None) -> int:
                 lat = _time(call, flush, args.steps)
                 res = _result(op, lat, _device_busy(call))
                 kernel = next(iter(op.iter_kernels()), None) if hasattr(op, "iter_kernels") else None
-                params = {"label": row["label"], "q_shape": tuple(row["q_shape"]), "kv_shape": tuple(row["kv_shape"]), "dtype": dname,
-                          "kv_dtype": row.get("kv_dtype", dname)}
+                if "q_shape" in row:
+                    params = {"label": row["label"], "q_shape": tuple(row["q_shape"]), "kv_shape": tuple(row["kv_shape"]), "dtype": dname,
+                              "kv_dtype": row.get("kv_dtype", dname)}
+                else:
+                    params = {"label": row["label"], "total_q": row["total_q"], "batch": row["batch"], "heads": row["heads"],
+                              "heads_kv": row["heads_kv"], "dim": row["dim"], "dtype": dname, "kv_dtype": row.get("cache_dtype", dname)}
                 if "page_size" in row:
                     params["page_size"] = row["page_size"]
                 report.record(op_name, params, res, "tileops", getattr(kernel, "config", None))

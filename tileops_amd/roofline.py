@@ -96,3 +96,42 @@ def gqa_decode_roofline(op: Optional[Any] = None, **kwargs: Any) -> tuple[int, i
     b = algorithmic_bytes(sum_len=seen["sum_len"], sum_pages=0, batch=batch, q_len=1, heads=heads, heads_kv=heads_kv,
                           dim=dim, q_bytes=q_bytes, kv_bytes=seen["kv_bytes"], fp8_scales=seen["fp8"])
     return algorithmic_flops(sum_len=seen["sum_len"], q_len=1, heads=heads, dim=dim), b["total"] - 4 * batch
+
+
+def _distribute_total(total: int, batch: int, max_len: int) -> list[int]:
+    """src/tileops/perf/formulas.py:467-475."""
+    lengths, remaining = [0] * batch, total
+    for idx in range(batch):
+        value = min(max_len, remaining - (batch - idx - 1))
+        lengths[idx] = value
+        remaining -= value
+    return lengths
+
+
+def gqa_prefill_paged_with_kv_cache_fwd_roofline(op: Optional[Any] = None, **kwargs: Any) -> tuple[int, int]:
+    """Paged-cache GQA prefill: the reference's conservative model (src/tileops/perf/formulas.py:532-587) -- visible
+    score count from per-request ``q_lens`` / ``cache_lens`` (a deterministic fill when a workload row omits them);
+    bytes = Q, old K/V, new K/V read, new K/V appended, O, and the metadata, all at the attention element size."""
+    d = _fields(op, kwargs)
+    batch, heads, heads_kv, dim = int(d["batch"]), int(d["heads"]), int(d["heads_kv"]), int(d["dim"])
+    max_pages, page = int(d["max_pages_per_req"]), int(d["page_size"])
+    max_q = int(d.get("max_seqlen_q") or max_pages * page)
+    causal = bool(d.get("is_causal", True))
+    elem = _itemsize(d.get("dtype") or d.get("dtypes") or "float16")
+    q_lens = d.get("q_lens")
+    total_q = int(d["total_q"]) if d.get("total_q") is not None else (int(sum(q_lens)) if q_lens is not None else batch * max_q)
+    if q_lens is None:
+        q_lens = _distribute_total(total_q, batch, max_q)
+    cache_lens = d.get("cache_lens")
+    if cache_lens is None:
+        cap = max_pages * page if d.get("max_position") is None else int(d["max_position"])
+        cache_lens = [max(cap - int(n), 0) for n in q_lens]
+    visible = old = 0
+    for n, m in zip(q_lens, cache_lens):
+        n, m = int(n), int(m)
+        old += m
+        visible += n * m + n * (n + 1) // 2 if causal else n * (m + n)
+    q_elems = total_q * heads * dim
+    new_kv = 2 * total_q * heads_kv * dim
+    nbytes = (q_elems + 2 * old * heads_kv * dim + new_kv + new_kv + q_elems) * elem + (batch + 1) * 4 + batch * 4 + batch * max_pages * 4
+    return int(4 * heads * visible * dim), int(nbytes)
