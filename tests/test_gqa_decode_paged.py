@@ -466,3 +466,51 @@ def test_graph_capture_and_replay_with_changing_cache_contents(fp8):
         assert torch.isfinite(eager).all()
         assert torch.equal(out_g, eager), f"replay {it} differs from the eager call"
         assert torch.equal(eager, eager0) == (it == 0)
+
+
+def _random_configs(n, seed):
+    """Seeded draw of small shapes over everything the ops accept: head counts and groups, head_dim, page size, query
+    tokens, dtype, FP8 cache, softcap, custom scale (also negative), causal or not, ragged lengths with zeros."""
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=g))]  # noqa: E731
+    out = []
+    for i in range(n):
+        heads_kv = pick([1, 2, 4, 8])
+        group = pick([1, 2, 3, 4, 5, 8, 16])
+        dim = pick([128, 128, 128, 64, 256])
+        page = pick([16, 32, 64, 128, 48] if dim != 128 else [16, 32, 64, 128])
+        q_len = pick([1, 1, 1, 2, 3, 5, 8, 11])
+        batch = pick([1, 2, 3, 7])
+        lens = [int(torch.randint(0, 900, (1,), generator=g)) for _ in range(batch)]
+        lens = [max(n_, q_len) if n_ > 0 else 0 for n_ in lens]
+        out.append(dict(i=i, heads_kv=heads_kv, heads=heads_kv * group, dim=dim, page=page, q_len=q_len, lens=lens,
+                        dtype=pick([torch.bfloat16, torch.float16]), fp8=pick([False, False, True]),
+                        softcap=pick([0.0, 0.0, 0.0, 5.0, 30.0]), sm_scale=pick([None, None, None, 0.05, -0.11, 0.3]),
+                        causal=pick([True, True, False])))
+    return out
+
+
+@pytest.mark.parametrize("cfg", _random_configs(48, seed=2024), ids=lambda c: f"r{c['i']}")
+def test_random_shapes_against_the_oracle_on_every_kernel_that_serves_them(cfg):
+    require_gfx950()
+    c = cfg
+    case = _ragged_case(len(c["lens"]), c["heads"], c["heads_kv"], c["dim"], c["page"], c["lens"], c["dtype"], q_len=c["q_len"],
+                        fp8=c["fp8"], seed=100 + c["i"])
+    n_kv = case[1].shape[0]
+    tol = 3e-2 if c["fp8"] else 2e-2
+    ran = 0
+    for key in KERNELS:
+        if c["q_len"] == 1:
+            op = PagedOp(len(c["lens"]), c["heads"], c["heads_kv"], n_kv, c["dim"], c["page"], sm_scale=c["sm_scale"], softcap=c["softcap"] or None)
+        else:
+            op = MultiOp(len(c["lens"]), c["q_len"], c["heads"], c["heads_kv"], n_kv, c["dim"], c["page"], is_causal=c["causal"],
+                         sm_scale=c["sm_scale"], softcap=c["softcap"] or None)
+        if not _serves(op, key, c["dtype"], c["fp8"]):
+            continue
+        _force(op, key)
+        kw = dict(sm_scale=c["sm_scale"], softcap=c["softcap"])
+        if c["q_len"] > 1:
+            kw["is_causal"] = c["causal"]
+        _run_and_compare(op, case, c["page"], tol, **kw)
+        ran += 1
+    assert ran >= 1
