@@ -107,9 +107,6 @@ __device__ __forceinline__ const char* uni_ptr(const char* p) {
 // LDS-DMA wait state and the five wait states a VMEM instruction needs after a VALU write of its SGPR base,
 // which the compiler's hazard recogniser cannot insert inside an asm block.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const char* sbase) {
-#ifdef MI355_DEBUG_NO_DMA
-  return;
-#endif
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   sbase = uni_ptr(sbase);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
@@ -218,6 +215,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   // a sequence) spread over all L2s and memory channels; renumbering them XCD-contiguously measured slower.
 #ifdef MI355_PHASE_TIMERS
   const uint64_t tm_kernel0 = __builtin_readcyclecounter();
+  const uint64_t tm_wall0 = wall_clock64();  // constant 100 MHz, common to all XCDs (the cycle counter is per XCD clock)
 #endif
   const int gw = blockIdx.x * NW + wave;
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
@@ -524,14 +522,6 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       for (int db = 0; db < 8; db++) va_op[db] = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
     }
     if (!FP8) __builtin_amdgcn_sched_barrier(0);
-#ifdef MI355_ABL_NO_LDS
-#pragma unroll
-    for (int tb = 0; tb < 2; tb++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) ka_op[tb][j] = qreg[0][j];
-#pragma unroll
-    for (int db = 0; db < 8; db++) va_op[db] = qreg[0][db & 3];
-#endif
     // ---- S^T = K . Q^T : the two 16-token blocks interleaved so dependent MFMAs are one apart -------------
     f32x4 s_acc[2][NRB];
 #pragma unroll
@@ -544,11 +534,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
         for (int tb = 0; tb < 2; tb++) {
-#ifndef MI355_ABL_NO_QK
           s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
-#else
-          s_acc[tb][rb][j] += __uint_as_float(ka_op[tb][j][0]);
-#endif
         }
     // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
     const bool need_mask = tok0 + kCT > cu.len - qoff;
@@ -581,12 +567,6 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
           for (int i = 0; i < 4; i++)
             if (tok0 + 16 * tb + 4 * g + i >= limit[rb]) x[tb][i] = -INFINITY;
       }
-#ifdef MI355_ABL_NO_SOFTMAX
-      alpha[rb] = 1.f;
-      pk[rb][0] = __float_as_uint(x[0][0]); pk[rb][1] = __float_as_uint(x[0][2]); pk[rb][2] = __float_as_uint(x[1][0]); pk[rb][3] = __float_as_uint(x[1][3]);
-      l_run[rb] += x[0][1];
-      continue;
-#endif
       float mt = max2(max3(x[0][0], x[0][1], x[0][2]), max3(x[0][3], x[1][0], max3(x[1][1], x[1][2], x[1][3])));
       mt = group_max(mt) * exp_scale;
       // Lazy rescale: the running reference m_run only moves when the tile maximum exceeds it by more than
@@ -629,11 +609,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     for (int db = 0; db < 8; db++)
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++) {
-#ifndef MI355_ABL_NO_PV
         o_acc[rb][db] = Mma<QT>::run(va_op[db], pk[rb], o_acc[rb][db]);
-#else
-        o_acc[rb][db][0] += __uint_as_float(va_op[db][0] ^ pk[rb][0]);
-#endif
       }
   };
 
@@ -697,7 +673,6 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     else wait_vmcnt<0>();
   };
   auto run_score_step = [&](int ring) __attribute__((always_inline)) -> bool {
-#ifndef MI355_DEBUG_NO_COMPUTE
     if constexpr (NRB == 1) {
       // one copy of the body per ring slot: the slot offset folds into the LDS read immediates
       if (ring == 0) return score_step(0u, cc);
@@ -707,17 +682,10 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     } else {
       return score_step((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
     }
-#else
-    return false;
-#endif
-  };
-  auto run_value_step = [&]() __attribute__((always_inline)) {
-#ifndef MI355_DEBUG_NO_COMPUTE
-    value_step();
-#endif
   };
 #ifdef MI355_PHASE_TIMERS
-  // measurement build only: per-wave cycle totals of the loop phases, left behind the workspace proper
+  // Measurement build only (-DMI355_PHASE_TIMERS, see tileops_amd/perf/phase_timers.py): per-wave cycle totals of the
+  // loop phases and wall-clock start/end stamps, eight floats per wave written behind the workspace proper.
   uint64_t tm_issue = 0, tm_wait = 0, tm_comp = 0, tm_seg = 0, tm_mark = __builtin_readcyclecounter();
   const uint64_t tm_loop0 = tm_mark;
 #define TM(acc) { uint64_t now_ = __builtin_readcyclecounter(); acc += now_ - tm_mark; tm_mark = now_; }
@@ -742,7 +710,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
         TM(tm_wait)
         moved = run_score_step(ring);
         if (__builtin_expect(moved, 0)) break;
-        run_value_step();
+        value_step();
         TM(tm_comp)
         ++u;
         ++cc.j;
@@ -750,7 +718,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       }
       if (moved) {  // rare after the first tiles of a sequence: finish this tile out of line, then re-enter
         rescale();
-        run_value_step();
+        value_step();
         TM(tm_comp)
         ++u;
         ++cc.j;
@@ -768,7 +736,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   if (lane == 0) {
     float* dst = (float*)(ws_prefix + ((p.batch + 1) * 4 + 63) / 64 * 64) + (size_t)gw * 8;  // past the records: caller over-allocates
     dst[0] = (float)tm_issue; dst[1] = (float)tm_wait; dst[2] = (float)tm_comp; dst[3] = (float)tm_seg;
-    dst[4] = (float)(tm_loop0 - tm_kernel0); dst[5] = (float)(tm_mark - tm_kernel0); dst[6] = (float)n_units; dst[7] = (float)seg_count;
+    dst[4] = (float)(tm_loop0 - tm_kernel0); dst[5] = (float)(tm_mark - tm_kernel0);
+    dst[6] = (float)(tm_wall0 & 0xFFFFFF); dst[7] = (float)(wall_clock64() & 0xFFFFFF);
   }
 #endif
 #undef TM
