@@ -240,3 +240,16 @@ def test_prefill_rejects_bad_calls():
     bad[3] = case[3].to(torch.bfloat16)
     with pytest.raises(ValueError, match="Expected k_pages.dtype"):
         op(*bad, 4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fp8", [False, True])
+def test_llama_shape_chunks_of_hundreds_of_rows_against_long_prefixes(fp8):
+    """The reference's llama-8b workload shape at reduced batch (attention.yaml:296): 32/8 heads, head_dim 128, page 64,
+    chunks of 512 and 300 rows against prefixes of 4096 and 1000 tokens -- dozens of row groups per kv head, prefixes
+    spanning many partitions, a chunk that ends mid-page."""
+    require_gfx950()
+    q_lens, old_lens = [512, 300], [4096, 1000]
+    case = _case(q_lens, old_lens, 32, 8, 128, torch.float16, fp8=fp8, page=64, max_pages=72, seed=21)
+    op = PrefillOp(batch=2, heads=32, heads_kv=8, max_pages_per_req=72, page_size=64, dim=128, cache_dtype=FP8 if fp8 else None)
+    _run(op, case, 64, torch.float16, fp8=fp8)
