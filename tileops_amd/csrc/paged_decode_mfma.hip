@@ -44,6 +44,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
+constexpr int kSharedStages = 4;  // ring depth of the pair-shared fp8 variant (8.25 KiB a stage, four pairs: 132 KiB)
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
@@ -202,10 +203,17 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 }
 
 // ------------------------------------------------------------------------------------------------------
-template <typename QT, typename KVT, int NRB, int NS, int NW>
-__global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+// SH (pair-shared stages): with two or more row groups per kv head, waves 2m and 2m+1 of a workgroup serve row groups
+// 2m', 2m'+1 of the same (partition, kv head), i.e. they walk the same tiles.  They then share one LDS ring: each
+// fetches half of every stage, and one workgroup barrier per tile makes both halves visible and retires the slot
+// that is refilled next.  The launcher only takes this variant when every wave of a workgroup belongs to the same
+// partition, so all of them execute the same number of barriers.
+template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
+__global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
+  constexpr int NIW = SH ? G::NI / 2 : G::NI;          // K (or V) fetch instructions per stage issued by this wave
+  constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63;
@@ -309,7 +317,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
 
   // ---- loop-invariant lane constants ------------------------------------------------------------------
   const uint32_t row_stride = (uint32_t)p.heads_kv * G::ROW;  // bytes between consecutive tokens of the pool
-  const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + wave * (NS * G::STAGE);
+  const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + (SH ? wave >> 1 : wave) * (NS * G::STAGE);
+  const int half = SH ? (rg & 1) : 0;  // which half of every stage this wave fetches
 
   // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
   // t = i*TPI + l/LPT (LPT lanes per token row), 16-byte slot l%LPT of that row.  The chunk fetched into
@@ -329,7 +338,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
 #pragma unroll
     for (int v = 0; v < 2; v++) voff_k[v] = ts * row_stride + ((slot ^ ((4 * v + ts / 2) & 7)) << 4);
 #pragma unroll
-    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (((ts / 2) & 3) + 4 * v)) << 4);
+    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (((ts / 2) & 3) + 4 * (SH ? half : v))) << 4);
   }
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
@@ -373,7 +382,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   auto issue = [&](const Cursor& cu, int slot_idx) __attribute__((always_inline)) {
     const int tok0 = cu.j * kCT;
     const int nvalid = min(kCT, cu.len - tok0);  // >= 1
-    const uint32_t lds = lds_wave + slot_idx * G::STAGE;
+    const uint32_t lds = lds_wave + slot_idx * G::STAGE + half * (NIW * 1024);
     int64_t ptok0, ptok1 = 0;  // physical token of the stage's first token (and of its second 16-token page)
     if (ps16) {
       int last_pg = (cu.len - 1) >> 4;
@@ -388,11 +397,12 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     }
     if (nvalid == kCT && !ps16) {
       // common case: 32 valid tokens inside one page -- straight-line, two scalar adds per instruction
-      const char* kb = kpool + ptok0 * row_stride;
-      const char* vb = vpool + ptok0 * row_stride;
+      const int64_t ptok = ptok0 + half * (NIW * G::TPI);
+      const char* kb = kpool + ptok * row_stride;
+      const char* vb = vpool + ptok * row_stride;
       const uint32_t step = G::TPI * row_stride;
 #pragma unroll
-      for (int i = 0; i < G::NI; i++) {
+      for (int i = 0; i < NIW; i++) {
         dma16_nt(lds + i * 1024, voff_k[FP8 ? (i & 1) : (i & 3)], kb + i * step);
         dma16_nt(lds + G::KBYTES + i * 1024, voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)], vb + i * step);
       }
@@ -402,11 +412,11 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
       constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
 #pragma unroll
-      for (int i = 0; i < G::NI; i++) {
-        int si = min(i, i_last);
+      for (int i = 0; i < NIW; i++) {
+        int si = min(i + half * NIW, i_last);
         int64_t ptok = ps16 ? (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI : ptok0 + si * G::TPI;
         uint32_t vk = voff_k[FP8 ? (i & 1) : (i & 3)], vv = voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)];
-        if (si == i_last && ts > t_last) {
+        if (si == i_last && ts > t_last) {  // (also every instruction past i_last: si is clamped)
           uint32_t back = (uint32_t)(ts - t_last) * row_stride;
           vk -= back;
           vv -= back;
@@ -419,7 +429,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       int tk = min(lane & 31, nvalid - 1);
       int64_t ptok = ps16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
       const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + (p.scale_per_tensor ? 0 : ptok * p.heads_kv + kvh);
-      dma4(lds + 2 * G::KBYTES, sp);
+      dma4(lds_wave + slot_idx * G::STAGE + 2 * G::KBYTES, sp);  // (both waves of a pair: same bytes, same place)
     }
   };
 
@@ -476,7 +486,11 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   // value_step: O^T += V^T.P^T.  Between them the caller rescales the accumulators when asked to -- outside the
   // steady-state loop, because the accumulators live in accumulation registers that the vector ALU cannot
   // address, and a rescale inside the loop makes the register allocator shuttle all of them on every iteration.
-  u32x4 va_op[8];
+  // With an fp8 cache and several row blocks registers are short: V^T then stays in bytes until the PV product
+  // consumes it (widened one 16-column block at a time, in between the MFMAs).
+  constexpr bool LATE_V = FP8 && NRB >= 2;
+  u32x4 va_op[LATE_V ? 1 : 8];
+  i32x2 vraw[LATE_V ? 8 : 1];
   u32x4 pk[NRB];
   float alpha[NRB];
   auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
@@ -498,7 +512,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
       }
     } else {
       u32x4 kraw[2][2];
-      i32x2 vraw[8];
+      i32x2 vnow[8];
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
@@ -509,7 +523,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
         vsc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 128 + 64 * tb));
       }
 #pragma unroll
-      for (int db = 0; db < 8; db++) vraw[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
+      for (int db = 0; db < 8; db++) vnow[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
@@ -519,7 +533,10 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
           ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
         }
 #pragma unroll
-      for (int db = 0; db < 8; db++) va_op[db] = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
+      for (int db = 0; db < 8; db++) {
+        if constexpr (LATE_V) vraw[db] = vnow[db];
+        else va_op[db] = widen8<QT>((uint32_t)vnow[db][0], (uint32_t)vnow[db][1]);
+      }
     }
     if (!FP8) __builtin_amdgcn_sched_barrier(0);
     // ---- S^T = K . Q^T : the two 16-token blocks interleaved so dependent MFMAs are one apart -------------
@@ -606,11 +623,13 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   };
   auto value_step = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int db = 0; db < 8; db++)
+    for (int db = 0; db < 8; db++) {
+      u32x4 vt;
+      if constexpr (LATE_V) vt = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
+      else vt = va_op[db];
 #pragma unroll
-      for (int rb = 0; rb < NRB; rb++) {
-        o_acc[rb][db] = Mma<QT>::run(va_op[db], pk[rb], o_acc[rb][db]);
-      }
+      for (int rb = 0; rb < NRB; rb++) o_acc[rb][db] = Mma<QT>::run(vt, pk[rb], o_acc[rb][db]);
+    }
   };
 
   auto end_segment = [&](const Cursor& cu, bool complete, int which) __attribute__((always_inline)) {
@@ -667,9 +686,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   };
   auto wait_stage = [&](int u) __attribute__((always_inline)) {
     const int ahead = issued - u - 1;  // stages issued after the one consumed now
-    if (ahead >= 3) wait_vmcnt<(NS > 3 ? 3 : NS - 1) * G::IPS>();
-    else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * G::IPS>();
-    else if (ahead == 1) wait_vmcnt<G::IPS>();
+    if (ahead >= 3) wait_vmcnt<(NS > 3 ? 3 : NS - 1) * IPSW>();
+    else if (ahead == 2) wait_vmcnt<(NS > 2 ? 2 : NS - 1) * IPSW>();
+    else if (ahead == 1) wait_vmcnt<IPSW>();
     else wait_vmcnt<0>();
   };
   auto run_score_step = [&](int ring) __attribute__((always_inline)) -> bool {
@@ -696,7 +715,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
   while (u < n_units) {
     const int seg_first_j = cc.j;
     const int seg_units = min(cc.nt - cc.j, n_units - u);
-    issue_ahead(ring);   // before the query loads, so the next tile is already in flight while they land
+    if (!SH) issue_ahead(ring);  // before the query loads, so the next tile is already in flight while they land
     TM(tm_issue)
     begin_segment(cc);
     TM(tm_seg)
@@ -704,12 +723,26 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_mfma_kernel(const Decode
     while (k < seg_units) {
       bool moved = false;
       for (; k < seg_units; ++k) {  // steady state: no tile in here rescales the accumulators
-        if (k > 0) issue_ahead(ring);
+        if (!SH && k > 0) issue_ahead(ring);
         TM(tm_issue)
         wait_stage(u);
+        if (SH) {
+          // Own half of tile u has landed; past the barrier so has the partner's, and every wave of the workgroup
+          // has finished reading tile u-1, whose slot the next fetch overwrites.
+          asm volatile("s_barrier" ::: "memory");
+          TM(tm_wait)
+          issue_ahead(ring);
+          TM(tm_issue)
+        }
         TM(tm_wait)
         moved = run_score_step(ring);
-        if (__builtin_expect(moved, 0)) break;
+        if constexpr (FP8 && NRB == 2) {
+          // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
+          if (__builtin_expect(moved, 0)) rescale();
+          moved = false;
+        } else {
+          if (__builtin_expect(moved, 0)) break;
+        }
         value_step();
         TM(tm_comp)
         ++u;
@@ -856,17 +889,16 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
 template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB <= 2) ? 8 : 4; }
 
-template <typename QT, typename KVT, int NRB>
-const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
-  constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
+template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
+const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   const int grid = (int)((waves + NW - 1) / NW);
-  const size_t lds = (size_t)NW * NS * Geom<KVT>::STAGE;
-  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW>;
+  const size_t lds = (size_t)(SH ? NW / 2 : NW) * NS * Geom<KVT>::STAGE;
+  if (SH && (n_rg % 2 != 0 || (p.heads_kv * n_rg) % NW != 0)) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
+  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SH>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
-  static bool lds_opted_in[64] = {};
+  static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return "hipGetDevice failed";
   if (dev < 0 || dev >= 64 || !lds_opted_in[dev]) {
@@ -885,6 +917,25 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
+template <typename QT, typename KVT, int NRB>
+const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
+  // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
+  constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
+  if constexpr (Geom<KVT>::FP8 && NRB == 2) {
+    // Two or more row groups per kv head would each fetch the same K/V tiles: pair them up on one LDS ring (half the
+    // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.  A
+    // workgroup must not straddle partitions (its waves meet at one barrier per tile), hence the choice of its size.
+    const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
+    if (n_rg % 2 == 0) {
+      const int per_part = p.heads_kv * n_rg;
+      if (per_part % 8 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 8, true>(p, ws_prefix, skip_combine, s);
+      if (per_part % 4 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 4, true>(p, ws_prefix, skip_combine, s);
+      return launch_t4<QT, KVT, NRB, kSharedStages, 2, true>(p, ws_prefix, skip_combine, s);
+    }
+  }
+  return launch_t4<QT, KVT, NRB, NS, NW, false>(p, ws_prefix, skip_combine, s);
 }
 
 int row_blocks_for(int rows, bool fp8) { return rows <= 16 ? 1 : ((rows <= 32 || fp8) ? 2 : 4); }
