@@ -44,7 +44,8 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
-constexpr int kSharedStages = 4;  // ring depth of the pair-shared fp8 variant (8.25 KiB a stage, four pairs: 132 KiB)
+constexpr bool kLateIssueFp8 = true;
+constexpr int kSharedStages = 4;  // ring depth of the pair-shared fp8 variant (8.25 KiB a stage, four pairs a CU: 132 KiB)
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
@@ -169,6 +170,10 @@ __device__ __forceinline__ void cursor_load_lens(Cursor& c, const DecodeParams& 
   const int lane = threadIdx.x & 63;
   c.lens_base = base;
   c.lens = seq_len_of(p, min(base + lane, p.batch - 1));
+  // Land the load here.  Left to itself the compiler waits for it where the register is next read -- after the
+  // join with the path that did not load, i.e. on every pass -- and its wait (vmcnt 0) also drains every
+  // direct-to-LDS load in flight.  An empty asm that reads the register moves the wait into this rare block.
+  asm volatile("" : "+v"(c.lens));
 }
 
 __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bool ps16) {
@@ -203,15 +208,18 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 }
 
 // ------------------------------------------------------------------------------------------------------
-// SH (pair-shared stages): with two or more row groups per kv head, waves 2m and 2m+1 of a workgroup serve row groups
-// 2m', 2m'+1 of the same (partition, kv head), i.e. they walk the same tiles.  They then share one LDS ring: each
-// fetches half of every stage, and one workgroup barrier per tile makes both halves visible and retires the slot
-// that is refilled next.  The launcher only takes this variant when every wave of a workgroup belongs to the same
-// partition, so all of them execute the same number of barriers.
+// SH (pair-shared stages): with an even number of row groups per kv head, a workgroup is two waves that serve row
+// groups 2m, 2m+1 of the same (partition, kv head), i.e. they walk the same tiles.  They share one LDS ring: each
+// fetches half of every stage, and one barrier per tile makes both halves visible and retires the slot that is
+// refilled next.  Both waves execute the same number of barriers because they own the same tile range.  Pairs are
+// kept this small on purpose: a barrier over more waves makes all of them fetch, then all of them compute, in step.
 template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
 __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
+  // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
+  // or after it (a tile lands before the next is requested: fewer requests in flight per compute unit).
+  constexpr bool LATE = SH || (FP8 && NRB == 1 && kLateIssueFp8);
   constexpr int NIW = SH ? G::NI / 2 : G::NI;          // K (or V) fetch instructions per stage issued by this wave
   constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -230,9 +238,21 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   const int per_part = p.heads_kv * n_rg;
   // integer division runs on the vector ALU; pin the results to scalar registers so that everything derived
   // from them (pool base pointers, LDS bases) is scalar arithmetic
-  const int part = uni(gw / per_part);
-  const int kvh = uni((gw - part * per_part) / n_rg);
-  const int rg = uni(gw - part * per_part - kvh * n_rg);
+  int part_, slot_;
+  if constexpr (SH) {
+    // Workgroup g runs on XCD g % 8.  All pairs of a partition (its kv heads read the same pages, and share the
+    // 32-byte sectors of the scale rows) go to one XCD, i.e. one L2; neighbouring partitions to different ones.
+    static_assert(NW == 2, "a shared-stage workgroup is one pair of waves");
+    const int pairs = per_part >> 1, x = blockIdx.x & 7, y = blockIdx.x >> 3;
+    part_ = x + 8 * (y / pairs);
+    slot_ = 2 * (y % pairs) + wave;
+  } else {
+    part_ = gw / per_part;
+    slot_ = gw - part_ * per_part;
+  }
+  const int part = uni(part_);
+  const int kvh = uni(slot_ / n_rg);
+  const int rg = uni(slot_ - kvh * n_rg);
   const int64_t NP = p.n_parts;
   const bool ps16 = p.page_size == 16;
 
@@ -369,12 +389,15 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   // compiler-visible memory load (whose vmcnt wait would drain the direct-to-LDS pipeline); the register
   // is refilled once per 64 pages.
   int bt_reg = 0, bt_base = 0, bt_seq = -1;
+  int kvs_seq = -1;
+  int64_t kvs_val = 0;  // kv_starts[kvs_seq], fetched once per sequence
   auto phys_page = [&](const Cursor& cu, int pg) __attribute__((always_inline)) -> int64_t {
     if (cu.b != bt_seq || pg < bt_base || pg >= bt_base + 64) {
       bt_seq = cu.b;
       bt_base = pg;
       int last_pg = uni((cu.len - 1) / p.page_size);  // never read past the entries the sequence owns
       bt_reg = p.block_table[(int64_t)cu.b * p.bt_row_stride + min(pg + lane, last_pg)];
+      asm volatile("" : "+v"(bt_reg));  // wait for it here, not after the join (see cursor_load_lens)
     }
     int64_t e = __builtin_amdgcn_readlane(bt_reg, pg - bt_base);
     return e < 0 ? 0 : (e >= p.n_pages ? p.n_pages - 1 : e);
@@ -389,7 +412,11 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
       ptok0 = phys_page(cu, cu.pg) * 16;
       ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
     } else if (p.kv_starts) {
-      ptok0 = (int64_t)p.kv_starts[cu.b] + tok0;  // packed contiguous keys: sequence b starts at kv_starts[b]
+      if (cu.b != kvs_seq) {  // packed contiguous keys: sequence b starts at kv_starts[b]
+        kvs_seq = cu.b;
+        kvs_val = uni(p.kv_starts[cu.b]);
+      }
+      ptok0 = kvs_val + tok0;
     } else if (p.contig_stride) {
       ptok0 = (int64_t)cu.b * p.contig_stride + tok0;  // contiguous cache: no table, a tile never straddles anything
     } else {
@@ -715,7 +742,7 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   while (u < n_units) {
     const int seg_first_j = cc.j;
     const int seg_units = min(cc.nt - cc.j, n_units - u);
-    if (!SH) issue_ahead(ring);  // before the query loads, so the next tile is already in flight while they land
+    if (!LATE) issue_ahead(ring);  // before the query loads, so the next tile is already in flight while they land
     TM(tm_issue)
     begin_segment(cc);
     TM(tm_seg)
@@ -723,18 +750,17 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
     while (k < seg_units) {
       bool moved = false;
       for (; k < seg_units; ++k) {  // steady state: no tile in here rescales the accumulators
-        if (!SH && k > 0) issue_ahead(ring);
+        if (!LATE && k > 0) issue_ahead(ring);
         TM(tm_issue)
         wait_stage(u);
         if (SH) {
           // Own half of tile u has landed; past the barrier so has the partner's, and every wave of the workgroup
           // has finished reading tile u-1, whose slot the next fetch overwrites.
           asm volatile("s_barrier" ::: "memory");
-          TM(tm_wait)
-          issue_ahead(ring);
-          TM(tm_issue)
         }
         TM(tm_wait)
+        if (LATE) issue_ahead(ring);
+        TM(tm_issue)
         moved = run_score_step(ring);
         if constexpr (FP8 && NRB == 2) {
           // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
@@ -893,9 +919,10 @@ template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
 const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
-  const int grid = (int)((waves + NW - 1) / NW);
-  const size_t lds = (size_t)(SH ? NW / 2 : NW) * NS * Geom<KVT>::STAGE;
-  if (SH && (n_rg % 2 != 0 || (p.heads_kv * n_rg) % NW != 0)) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
+  // shared-stage variant: 8 XCDs x (pairs of a partition) x ceil(n_parts / 8); pairs of partitions past the last exit at once
+  const int grid = SH ? 8 * (p.heads_kv * n_rg / 2) * ((p.n_parts + 7) / 8) : (int)((waves + NW - 1) / NW);
+  const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT>::STAGE;
+  if (SH && (n_rg % 2 != 0 || NW != 2)) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
   auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SH>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
   static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
@@ -925,15 +952,9 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
   if constexpr (Geom<KVT>::FP8 && NRB == 2) {
     // Two or more row groups per kv head would each fetch the same K/V tiles: pair them up on one LDS ring (half the
-    // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.  A
-    // workgroup must not straddle partitions (its waves meet at one barrier per tile), hence the choice of its size.
+    // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.
     const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
-    if (n_rg % 2 == 0) {
-      const int per_part = p.heads_kv * n_rg;
-      if (per_part % 8 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 8, true>(p, ws_prefix, skip_combine, s);
-      if (per_part % 4 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 4, true>(p, ws_prefix, skip_combine, s);
-      return launch_t4<QT, KVT, NRB, kSharedStages, 2, true>(p, ws_prefix, skip_combine, s);
-    }
+    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 2, true>(p, ws_prefix, skip_combine, s);
   }
   return launch_t4<QT, KVT, NRB, NS, NW, false>(p, ws_prefix, skip_combine, s);
 }
