@@ -390,8 +390,9 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   // is refilled once per 64 pages.
   int bt_reg = 0, bt_base = 0, bt_seq = -1;
   int kvs_seq = -1;
-  int64_t kvs_val = 0;  // kv_starts[kvs_seq], fetched once per sequence
-  auto phys_page = [&](const Cursor& cu, int pg) __attribute__((always_inline)) -> int64_t {
+  uint32_t kvs_val = 0;  // kv_starts[kvs_seq], fetched once per sequence
+  const int last_page_id = (int)p.n_pages - 1;
+  auto phys_page = [&](const Cursor& cu, int pg) __attribute__((always_inline)) -> int {
     if (cu.b != bt_seq || pg < bt_base || pg >= bt_base + 64) {
       bt_seq = cu.b;
       bt_base = pg;
@@ -399,64 +400,77 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
       bt_reg = p.block_table[(int64_t)cu.b * p.bt_row_stride + min(pg + lane, last_pg)];
       asm volatile("" : "+v"(bt_reg));  // wait for it here, not after the join (see cursor_load_lens)
     }
-    int64_t e = __builtin_amdgcn_readlane(bt_reg, pg - bt_base);
-    return e < 0 ? 0 : (e >= p.n_pages ? p.n_pages - 1 : e);
+    int e = __builtin_amdgcn_readlane(bt_reg, pg - bt_base);
+    return min(max(e, 0), last_page_id);
   };
-  auto issue = [&](const Cursor& cu, int slot_idx) __attribute__((always_inline)) {
+  // Row of the pool (physical token) that holds the first token of cu's tile.  The pool has fewer than 2^31 rows
+  // (checked by the launcher).  Tiles inside one page, or one contiguous sequence, follow each other 32 rows apart,
+  // so the issue cursor only comes here at page and sequence borders.  Not used with 16-token pages.
+  const bool paged = !p.kv_starts && !p.contig_stride;
+  auto locate = [&](const Cursor& cu) __attribute__((always_inline)) -> uint32_t {
+    const int tok0 = cu.j * kCT;
+    if (p.kv_starts) {  // packed contiguous keys: sequence b starts at kv_starts[b]
+      if (cu.b != kvs_seq) {
+        kvs_seq = cu.b;
+        kvs_val = (uint32_t)uni(p.kv_starts[cu.b]);
+      }
+      return kvs_val + tok0;
+    }
+    if (p.contig_stride) return (uint32_t)cu.b * (uint32_t)p.contig_stride + tok0;  // contiguous cache: no table
+    return (uint32_t)phys_page(cu, cu.pg) * (uint32_t)p.page_size + cu.off;
+  };
+  // fp8 scales of a full tile: lane l fetches the K (l < 32) or V scale of token l % 32; everything but the tile's
+  // row is folded into a per-lane pointer once
+  const uint32_t scale_row_bytes = p.scale_per_tensor ? 0u : (uint32_t)p.heads_kv * 4u;
+  const char* const scale_lane = (const char*)(lane < 32 ? p.k_scale : p.v_scale) +
+                                 (p.scale_per_tensor ? 0 : ((int64_t)(lane & 31) * p.heads_kv + kvh) * 4);
+  auto issue = [&](const Cursor& cu, int slot_idx, uint32_t prow) __attribute__((always_inline)) {
     const int tok0 = cu.j * kCT;
     const int nvalid = min(kCT, cu.len - tok0);  // >= 1
-    const uint32_t lds = lds_wave + slot_idx * G::STAGE + half * (NIW * 1024);
-    int64_t ptok0, ptok1 = 0;  // physical token of the stage's first token (and of its second 16-token page)
-    if (ps16) {
-      int last_pg = (cu.len - 1) >> 4;
-      ptok0 = phys_page(cu, cu.pg) * 16;
-      ptok1 = phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
-    } else if (p.kv_starts) {
-      if (cu.b != kvs_seq) {  // packed contiguous keys: sequence b starts at kv_starts[b]
-        kvs_seq = cu.b;
-        kvs_val = uni(p.kv_starts[cu.b]);
-      }
-      ptok0 = kvs_val + tok0;
-    } else if (p.contig_stride) {
-      ptok0 = (int64_t)cu.b * p.contig_stride + tok0;  // contiguous cache: no table, a tile never straddles anything
-    } else {
-      ptok0 = phys_page(cu, cu.pg) * p.page_size + cu.off;
-    }
+    const uint32_t lds_stage = lds_wave + slot_idx * G::STAGE;
+    const uint32_t lds = lds_stage + half * (NIW * 1024);
     if (nvalid == kCT && !ps16) {
       // common case: 32 valid tokens inside one page -- straight-line, two scalar adds per instruction
-      const int64_t ptok = ptok0 + half * (NIW * G::TPI);
-      const char* kb = kpool + ptok * row_stride;
-      const char* vb = vpool + ptok * row_stride;
+      const uint64_t boff = (uint64_t)(prow + half * (NIW * G::TPI)) * row_stride;
+      const char* kb = kpool + boff;
+      const char* vb = vpool + boff;
       const uint32_t step = G::TPI * row_stride;
 #pragma unroll
       for (int i = 0; i < NIW; i++) {
         dma16_nt(lds + i * 1024, voff_k[FP8 ? (i & 1) : (i & 3)], kb + i * step);
         dma16_nt(lds + G::KBYTES + i * 1024, voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)], vb + i * step);
       }
-    } else {
-      // tail of a sequence and/or 16-token pages: rows past the valid ones re-read the last valid row, so
-      // nothing outside (block_table, real_seqlen_kv) is ever touched
-      const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
-      constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
+      if (FP8) dma4(lds_stage + 2 * G::KBYTES, scale_lane + (uint64_t)prow * scale_row_bytes);  // (both waves of a pair: same bytes, same place)
+      return;
+    }
+    // tail of a sequence and/or 16-token pages: rows past the valid ones re-read the last valid row, so
+    // nothing outside (block_table, real_seqlen_kv) is ever touched
+    int64_t ptok0 = prow, ptok1 = 0;  // physical token of the stage's first token (and of its second 16-token page)
+    if (ps16) {
+      int last_pg = (cu.len - 1) >> 4;
+      ptok0 = (int64_t)phys_page(cu, cu.pg) * 16;
+      ptok1 = (int64_t)phys_page(cu, min(cu.pg + 1, last_pg)) * 16;
+    }
+    const int i_last = (nvalid - 1) / G::TPI, t_last = (nvalid - 1) % G::TPI;
+    constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
 #pragma unroll
-      for (int i = 0; i < NIW; i++) {
-        int si = min(i + half * NIW, i_last);
-        int64_t ptok = ps16 ? (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI : ptok0 + si * G::TPI;
-        uint32_t vk = voff_k[FP8 ? (i & 1) : (i & 3)], vv = voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)];
-        if (si == i_last && ts > t_last) {  // (also every instruction past i_last: si is clamped)
-          uint32_t back = (uint32_t)(ts - t_last) * row_stride;
-          vk -= back;
-          vv -= back;
-        }
-        dma16_nt(lds + i * 1024, vk, kpool + ptok * row_stride);
-        dma16_nt(lds + G::KBYTES + i * 1024, vv, vpool + ptok * row_stride);
+    for (int i = 0; i < NIW; i++) {
+      int si = min(i + half * NIW, i_last);
+      int64_t ptok = ps16 ? (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI : ptok0 + si * G::TPI;
+      uint32_t vk = voff_k[FP8 ? (i & 1) : (i & 3)], vv = voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)];
+      if (si == i_last && ts > t_last) {  // (also every instruction past i_last: si is clamped)
+        uint32_t back = (uint32_t)(ts - t_last) * row_stride;
+        vk -= back;
+        vv -= back;
       }
+      dma16_nt(lds + i * 1024, vk, kpool + ptok * row_stride);
+      dma16_nt(lds + G::KBYTES + i * 1024, vv, vpool + ptok * row_stride);
     }
     if (FP8) {
       int tk = min(lane & 31, nvalid - 1);
       int64_t ptok = ps16 ? (tk < 16 ? ptok0 + tk : ptok1 + tk - 16) : ptok0 + tk;
       const float* sp = (lane < 32 ? p.k_scale : p.v_scale) + (p.scale_per_tensor ? 0 : ptok * p.heads_kv + kvh);
-      dma4(lds_wave + slot_idx * G::STAGE + 2 * G::KBYTES, sp);  // (both waves of a pair: same bytes, same place)
+      dma4(lds_stage + 2 * G::KBYTES, sp);
     }
   };
 
@@ -699,16 +713,22 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   // tiles of a segment.  The accumulators are initialised in the inner loop's preheader and stay in their
   // registers across it; issuing runs NS-1 tiles ahead of consumption and is oblivious to segment borders.
   Cursor ci = start, cc = start;
+  uint32_t ci_row = ps16 ? 0u : locate(ci);  // pool row of the tile at ci
   int issued = 0;
-  for (; issued < NS - 1 && issued < n_units; ++issued) {
-    issue(ci, issued);
+  auto advance = [&]() __attribute__((always_inline)) {  // ci to the next tile of the range (there is one)
     cursor_next(ci, p, ps16);
+    if (ps16) return;
+    if (ci.j == 0 || (paged && ci.off == 0)) ci_row = locate(ci);
+    else ci_row += kCT;
+  };
+  for (; issued < NS - 1 && issued < n_units;) {
+    issue(ci, issued, ci_row);
+    if (++issued < n_units) advance();
   }
   auto issue_ahead = [&](int ring) __attribute__((always_inline)) {
     if (issued < n_units) {
-      issue(ci, ring == 0 ? NS - 1 : ring - 1);  // the ring slot consumed in the previous iteration
-      cursor_next(ci, p, ps16);
-      ++issued;
+      issue(ci, ring == 0 ? NS - 1 : ring - 1, ci_row);  // the ring slot consumed in the previous iteration
+      if (++issued < n_units) advance();
     }
   };
   auto wait_stage = [&](int u) __attribute__((always_inline)) {
@@ -1014,6 +1034,9 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   p.part_o = (float*)ws;
   p.part_lse = (float*)(ws + align256(slots * kD * sizeof(float)));
   int* ws_prefix = (int*)(ws + align256(slots * kD * sizeof(float)) + align256(slots * sizeof(float)));
+  // the kernel addresses pool rows with 32 bits
+  const int64_t pool_rows = p.kv_starts ? INT32_MAX - 1 : (p.contig_stride ? (int64_t)p.batch * p.contig_stride : p.n_pages * p.page_size);
+  if (pool_rows >= INT32_MAX) return "MFMA kernel: the KV pool has 2^31 or more rows";
   if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag>(p, ws_prefix, skip_combine, s);
   if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag>(p, ws_prefix, skip_combine, s);
   if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag>(p, ws_prefix, skip_combine, s);
