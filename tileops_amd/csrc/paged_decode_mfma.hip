@@ -45,7 +45,7 @@ constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of 
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
 constexpr bool kLateIssueFp8 = true;
-constexpr int kSharedStages = 4;  // ring depth of the pair-shared fp8 variant (8.25 KiB a stage, four pairs a CU: 132 KiB)
+constexpr int kSharedStages = 4;  // ring depth of the pair-shared variants: fp8 8.25 KiB a stage x four pairs a CU, 16-bit 16 KiB x two pairs
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
@@ -214,7 +214,7 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // refilled next.  Both waves execute the same number of barriers because they own the same tile range.  Pairs are
 // kept this small on purpose: a barrier over more waves makes all of them fetch, then all of them compute, in step.
 template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
-__global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+__global__ __launch_bounds__(NW * 64, (SH && Geom<KVT>::FP8) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
@@ -970,7 +970,7 @@ template <typename QT, typename KVT, int NRB>
 const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
   constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
-  if constexpr (Geom<KVT>::FP8 && NRB == 2) {
+  if constexpr (NRB == 2) {
     // Two or more row groups per kv head would each fetch the same K/V tiles: pair them up on one LDS ring (half the
     // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.
     const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
@@ -979,7 +979,13 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   return launch_t4<QT, KVT, NRB, NS, NW, false>(p, ws_prefix, skip_combine, s);
 }
 
-int row_blocks_for(int rows, bool fp8) { return rows <= 16 ? 1 : ((rows <= 32 || fp8) ? 2 : 4); }
+// Row blocks (16 query rows each) per wave.  Above 32 rows an fp8 cache keeps two (its waves hold no accumulation
+// registers to spare); a 16-bit cache takes two when the row groups pair up on shared stages, else four.
+int row_blocks_for(int rows, bool fp8) {
+  if (rows <= 16) return 1;
+  if (rows <= 32 || fp8) return 2;
+  return ((rows + 31) / 32) % 2 == 0 ? 2 : 4;
+}
 
 template <typename QT, typename KVT>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {

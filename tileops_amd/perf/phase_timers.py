@@ -32,7 +32,11 @@ NAMES = ("issue", "wait", "compute", "segment", "prologue", "total")
 
 def _row_blocks(rows: int, fp8: bool) -> int:
     """Row blocks per wave the launcher picks (csrc/paged_decode_mfma.hip: row_blocks_for)."""
-    return 1 if rows <= 16 else (2 if (rows <= 32 or fp8) else 4)
+    if rows <= 16:
+        return 1
+    if rows <= 32 or fp8:
+        return 2
+    return 2 if ((rows + 31) // 32) % 2 == 0 else 4
 
 
 def run(name: str, hot: bool = False) -> None:
@@ -49,7 +53,7 @@ def run(name: str, hot: bool = False) -> None:
     nrb = _row_blocks(rows, fp8)
     n_rg = (rows + 16 * nrb - 1) // (16 * nrb)
     waves = nparts * cfg.heads_kv * n_rg
-    shared = fp8 and nrb == 2 and n_rg % 2 == 0  # wave pairs sharing an LDS ring (csrc/paged_decode_mfma.hip: launch_t3)
+    shared = nrb == 2 and n_rg % 2 == 0  # wave pairs sharing an LDS ring (csrc/paged_decode_mfma.hip: launch_t3)
     nw = 2 if shared else (8 if (fp8 and nrb <= 2) else 4)  # waves per workgroup
     if shared:
         waves = 2 * 8 * (cfg.heads_kv * n_rg // 2) * ((nparts + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
