@@ -92,10 +92,10 @@ __device__ __forceinline__ int64_t physical_token(const int32_t* __restrict__ bt
 template <bool SOFTCAP>
 __device__ __forceinline__ float to_logit2(float qk, float score_scale, float cap_log2e, float inv_cap_scale) {
   if (SOFTCAP) {
-    float z = qk * inv_cap_scale;
-    // tanh(z) = 1 - 2/(exp(2z)+1); exp2f saturates cleanly at both ends
-    float e = exp2f(z * (2.0f * 1.4426950408889634f));
-    float t = 1.0f - 2.0f / (e + 1.0f);
+    // tanh(z) = 1 - 2/(exp(2z)+1) on the raw hardware exp2 and reciprocal (1 ulp each): exp2 saturates to 0 or +inf
+    // and rcp(+inf) = 0, so both ends come out as exactly -1 and +1; the absolute error near zero is ~1e-7
+    float e = __builtin_amdgcn_exp2f(qk * (inv_cap_scale * (2.0f * 1.4426950408889634f)));
+    float t = __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(e + 1.0f), 1.0f);
     return cap_log2e * t;
   }
   return qk * score_scale;

@@ -238,21 +238,26 @@ __global__ __launch_bounds__(NW * 64, (SH && Geom<KVT>::FP8) ? 2 : 1) void paged
   const int per_part = p.heads_kv * n_rg;
   // integer division runs on the vector ALU; pin the results to scalar registers so that everything derived
   // from them (pool base pointers, LDS bases) is scalar arithmetic
-  int part_, slot_;
+  int part_, kvh_, rg_;
   if constexpr (SH) {
-    // Workgroup g runs on XCD g % 8.  All pairs of a partition (its kv heads read the same pages, and share the
-    // 32-byte sectors of the scale rows) go to one XCD, i.e. one L2; neighbouring partitions to different ones.
+    // Workgroup g runs on XCD g % 8.  The pairs of one (partition, kv head) read the same tiles and go to one XCD,
+    // i.e. one L2.  Such groups are numbered kv-head-major, so with many partitions the kv heads of a partition (same
+    // pages, shared 32-byte sectors of the scale rows) also meet on one XCD and neighbouring partitions land on
+    // different ones, while a call with few partitions still spreads over all eight.
     static_assert(NW == 2, "a shared-stage workgroup is one pair of waves");
-    const int pairs = per_part >> 1, x = blockIdx.x & 7, y = blockIdx.x >> 3;
-    part_ = x + 8 * (y / pairs);
-    slot_ = 2 * (y % pairs) + wave;
+    const int pairs = n_rg >> 1, x = blockIdx.x & 7, y = blockIdx.x >> 3;
+    const int gid = x + 8 * (y / pairs);
+    kvh_ = gid / p.n_parts;
+    part_ = kvh_ < p.heads_kv ? gid - kvh_ * p.n_parts : p.n_parts;  // groups past the last: leave below
+    rg_ = 2 * (y % pairs) + wave;
   } else {
     part_ = gw / per_part;
-    slot_ = gw - part_ * per_part;
+    kvh_ = (gw - part_ * per_part) / n_rg;
+    rg_ = gw - part_ * per_part - kvh_ * n_rg;
   }
   const int part = uni(part_);
-  const int kvh = uni(slot_ / n_rg);
-  const int rg = uni(slot_ - kvh * n_rg);
+  const int kvh = uni(kvh_);
+  const int rg = uni(rg_);
   const int64_t NP = p.n_parts;
   const bool ps16 = p.page_size == 16;
 
@@ -939,8 +944,9 @@ template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
 const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
-  // shared-stage variant: 8 XCDs x (pairs of a partition) x ceil(n_parts / 8); pairs of partitions past the last exit at once
-  const int grid = SH ? 8 * (p.heads_kv * n_rg / 2) * ((p.n_parts + 7) / 8) : (int)((waves + NW - 1) / NW);
+  // shared-stage variant: 8 XCDs x (pairs of a group) x ceil(groups / 8), a group being one (partition, kv head); the
+  // pairs of groups past the last exit at once
+  const int grid = SH ? 8 * (n_rg / 2) * ((p.n_parts * p.heads_kv + 7) / 8) : (int)((waves + NW - 1) / NW);
   const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT>::STAGE;
   if (SH && (n_rg % 2 != 0 || NW != 2)) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
   auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SH>;

@@ -56,7 +56,7 @@ def run(name: str, hot: bool = False) -> None:
     shared = nrb == 2 and n_rg % 2 == 0  # wave pairs sharing an LDS ring (csrc/paged_decode_mfma.hip: launch_t3)
     nw = 2 if shared else (8 if (fp8 and nrb <= 2) else 4)  # waves per workgroup
     if shared:
-        waves = 2 * 8 * (cfg.heads_kv * n_rg // 2) * ((nparts + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
+        waves = 2 * 8 * (n_rg // 2) * ((nparts * cfg.heads_kv + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
     ws = torch.zeros(nbytes + waves * 32 + 4096, dtype=torch.uint8, device=dev)
     flush_w = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     flush_r = torch.ones(128 << 20, dtype=torch.int32, device=dev)
