@@ -45,7 +45,6 @@ constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of 
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
 constexpr bool kLateIssueFp8 = true;
-constexpr int kSharedStages = 4;  // ring depth of the pair-shared variants: fp8 8.25 KiB a stage x four pairs a CU, 16-bit 16 KiB x two pairs
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
@@ -214,7 +213,7 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // refilled next.  Both waves execute the same number of barriers because they own the same tile range.  Pairs are
 // kept this small on purpose: a barrier over more waves makes all of them fetch, then all of them compute, in step.
 template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
-__global__ __launch_bounds__(NW * 64, (SH && Geom<KVT>::FP8) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+__global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
@@ -787,7 +786,7 @@ __global__ __launch_bounds__(NW * 64, (SH && Geom<KVT>::FP8) ? 2 : 1) void paged
         if (LATE) issue_ahead(ring);
         TM(tm_issue)
         moved = run_score_step(ring);
-        if constexpr (FP8 && NRB == 2) {
+        if constexpr (SH || (FP8 && NRB == 2)) {
           // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
           if (__builtin_expect(moved, 0)) rescale();
           moved = false;
@@ -938,6 +937,9 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
 // Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
+// Ring depth of the pair-shared variants, four pairs (eight waves) a compute unit: fp8 4 x 8.25 KiB, 16-bit 2 x 16 KiB a pair.
+template <typename KVT> constexpr int kSharedStages = Geom<KVT>::FP8 ? 4 : 2;
+
 template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB <= 2) ? 8 : 4; }
 
 template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
@@ -980,7 +982,7 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
     // Two or more row groups per kv head would each fetch the same K/V tiles: pair them up on one LDS ring (half the
     // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.
     const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
-    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, kSharedStages, 2, true>(p, ws_prefix, skip_combine, s);
+    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, kSharedStages<KVT>, 2, true>(p, ws_prefix, skip_combine, s);
   }
   return launch_t4<QT, KVT, NRB, NS, NW, false>(p, ws_prefix, skip_combine, s);
 }
@@ -1021,7 +1023,9 @@ int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
   const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
   // resident waves per CU: eight for the fp8 single-row-block kernel (LDS-limited, ~160 VGPRs), otherwise four
   // (LDS-limited with a 16-bit cache, register-limited -- one wave per SIMD -- with more than one row block)
-  const int waves_per_cu = (kv_dtype == MI355_DT_FP8_E4M3FN && nrb <= 2) ? 8 : 4;
+  // -- and eight again for wave pairs on shared stages, which keep their accumulators in ordinary vector registers
+  const bool shared = nrb == 2 && n_rg % 2 == 0;
+  const int waves_per_cu = ((kv_dtype == MI355_DT_FP8_E4M3FN && nrb <= 2) || shared) ? 8 : 4;
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
