@@ -207,19 +207,20 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 }
 
 // ------------------------------------------------------------------------------------------------------
-// SH (pair-shared stages): with an even number of row groups per kv head, a workgroup is two waves that serve row
-// groups 2m, 2m+1 of the same (partition, kv head), i.e. they walk the same tiles.  They share one LDS ring: each
-// fetches half of every stage, and one barrier per tile makes both halves visible and retires the slot that is
-// refilled next.  Both waves execute the same number of barriers because they own the same tile range.  Pairs are
-// kept this small on purpose: a barrier over more waves makes all of them fetch, then all of them compute, in step.
-template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
-__global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+// SHW > 1 (shared stages): when the row groups of a kv head come in multiples of SHW, a workgroup is SHW waves that
+// serve SHW consecutive row groups of the same (partition, kv head), i.e. they walk the same tiles.  They share one
+// LDS ring: each fetches 1/SHW of every stage, and one barrier per tile makes all parts visible and retires the slot
+// that is refilled next.  All waves execute the same number of barriers because they own the same tile range.
+template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW>
+__global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT>;
   constexpr bool FP8 = G::FP8;
+  constexpr bool SH = SHW > 1;
+  static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
   // or after it (a tile lands before the next is requested: fewer requests in flight per compute unit).
   constexpr bool LATE = SH || (FP8 && NRB == 1 && kLateIssueFp8);
-  constexpr int NIW = SH ? G::NI / 2 : G::NI;          // K (or V) fetch instructions per stage issued by this wave
+  constexpr int NIW = G::NI / SHW;                     // K (or V) fetch instructions per stage issued by this wave
   constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -239,16 +240,15 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   // from them (pool base pointers, LDS bases) is scalar arithmetic
   int part_, kvh_, rg_;
   if constexpr (SH) {
-    // Workgroup g runs on XCD g % 8.  The pairs of one (partition, kv head) read the same tiles and go to one XCD,
+    // Workgroup g runs on XCD g % 8.  The workgroups of one (partition, kv head) read the same tiles and go to one XCD,
     // i.e. one L2.  Such groups are numbered kv-head-major, so with many partitions the kv heads of a partition (same
     // pages, shared 32-byte sectors of the scale rows) also meet on one XCD and neighbouring partitions land on
     // different ones, while a call with few partitions still spreads over all eight.
-    static_assert(NW == 2, "a shared-stage workgroup is one pair of waves");
-    const int pairs = n_rg >> 1, x = blockIdx.x & 7, y = blockIdx.x >> 3;
-    const int gid = x + 8 * (y / pairs);
+    const int per_group = n_rg / SHW, x = blockIdx.x & 7, y = blockIdx.x >> 3;  // workgroups per (partition, kv head)
+    const int gid = x + 8 * (y / per_group);
     kvh_ = gid / p.n_parts;
     part_ = kvh_ < p.heads_kv ? gid - kvh_ * p.n_parts : p.n_parts;  // groups past the last: leave below
-    rg_ = 2 * (y % pairs) + wave;
+    rg_ = SHW * (y % per_group) + wave;
   } else {
     part_ = gw / per_part;
     kvh_ = (gw - part_ * per_part) / n_rg;
@@ -341,8 +341,8 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
 
   // ---- loop-invariant lane constants ------------------------------------------------------------------
   const uint32_t row_stride = (uint32_t)p.heads_kv * G::ROW;  // bytes between consecutive tokens of the pool
-  const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + (SH ? wave >> 1 : wave) * (NS * G::STAGE);
-  const int half = SH ? (rg & 1) : 0;  // which half of every stage this wave fetches
+  const uint32_t lds_wave = uni((uint32_t)(size_t)LDS_PTR(char, smem)) + (SH ? 0 : wave) * (NS * G::STAGE);
+  const int i0 = SH ? wave * NIW : 0;  // first of the NIW K (and V) fetch instructions of a stage that this wave issues
 
   // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
   // t = i*TPI + l/LPT (LPT lanes per token row), 16-byte slot l%LPT of that row.  The chunk fetched into
@@ -350,20 +350,24 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
   //   bf16 K: f = t%16          bf16 V: f = 2*(t%8)
   //   fp8  K: f = (t/2)%8       fp8  V: f = (t/2)%4 + 4*((t/16)%2)
   constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
-  constexpr int NKV = FP8 ? 2 : 4;  // distinct per-lane offset patterns of the K instructions
+  // The patterns repeat every 4 (bf16 K), 2 (bf16 V, fp8 K) instructions, or change once half way (fp8 V): a wave
+  // keeps one offset register per distinct pattern among the instructions it issues.
   const int ts = lane / LPT, slot = lane % LPT;
-  uint32_t voff_k[NKV], voff_v[2];
-  if (!FP8) {
+  constexpr int NKO = NIW < (FP8 ? 2 : 4) ? NIW : (FP8 ? 2 : 4);
+  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (NIW < 2 ? NIW : 2);
+  uint32_t voff_k[NKO], voff_v[NVO];
 #pragma unroll
-    for (int v = 0; v < 4; v++) voff_k[v] = ts * row_stride + ((slot ^ ((4 * v + ts) & 15)) << 4);
-#pragma unroll
-    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (2 * ((4 * v + ts) & 7))) << 4);
-  } else {
-#pragma unroll
-    for (int v = 0; v < 2; v++) voff_k[v] = ts * row_stride + ((slot ^ ((4 * v + ts / 2) & 7)) << 4);
-#pragma unroll
-    for (int v = 0; v < 2; v++) voff_v[v] = ts * row_stride + ((slot ^ (((ts / 2) & 3) + 4 * (SH ? half : v))) << 4);
+  for (int e = 0; e < NKO; e++) {
+    const int i = i0 + e;
+    voff_k[e] = ts * row_stride + (FP8 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((4 * i + ts) & 15)) << 4));
   }
+#pragma unroll
+  for (int e = 0; e < NVO; e++) {
+    const int i = FP8 ? (NIW == 4 ? 2 * e : i0) : i0 + e;
+    voff_v[e] = ts * row_stride + (FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4) : ((slot ^ (2 * ((4 * i + ts) & 7))) << 4));
+  }
+  auto k_sel = [](int ii) __attribute__((always_inline)) { return ii % NKO; };
+  auto v_sel = [](int ii) __attribute__((always_inline)) { return FP8 ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
   constexpr int NKA = FP8 ? 2 : 4;
@@ -432,19 +436,19 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
     const int tok0 = cu.j * kCT;
     const int nvalid = min(kCT, cu.len - tok0);  // >= 1
     const uint32_t lds_stage = lds_wave + slot_idx * G::STAGE;
-    const uint32_t lds = lds_stage + half * (NIW * 1024);
+    const uint32_t lds = lds_stage + i0 * 1024;
     if (nvalid == kCT && !ps16) {
       // common case: 32 valid tokens inside one page -- straight-line, two scalar adds per instruction
-      const uint64_t boff = (uint64_t)(prow + half * (NIW * G::TPI)) * row_stride;
+      const uint64_t boff = (uint64_t)(prow + i0 * G::TPI) * row_stride;
       const char* kb = kpool + boff;
       const char* vb = vpool + boff;
       const uint32_t step = G::TPI * row_stride;
 #pragma unroll
       for (int i = 0; i < NIW; i++) {
-        dma16_nt(lds + i * 1024, voff_k[FP8 ? (i & 1) : (i & 3)], kb + i * step);
-        dma16_nt(lds + G::KBYTES + i * 1024, voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)], vb + i * step);
+        dma16_nt(lds + i * 1024, voff_k[k_sel(i)], kb + i * step);
+        dma16_nt(lds + G::KBYTES + i * 1024, voff_v[v_sel(i)], vb + i * step);
       }
-      if (FP8) dma4(lds_stage + 2 * G::KBYTES, scale_lane + (uint64_t)prow * scale_row_bytes);  // (both waves of a pair: same bytes, same place)
+      if (FP8) dma4(lds_stage + 2 * G::KBYTES, scale_lane + (uint64_t)prow * scale_row_bytes);  // (every wave of a ring: same bytes, same place)
       return;
     }
     // tail of a sequence and/or 16-token pages: rows past the valid ones re-read the last valid row, so
@@ -459,9 +463,9 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
     constexpr int IPP = 16 / G::TPI;  // instructions per 16-token page
 #pragma unroll
     for (int i = 0; i < NIW; i++) {
-      int si = min(i + half * NIW, i_last);
+      int si = min(i + i0, i_last);
       int64_t ptok = ps16 ? (si < IPP ? ptok0 : ptok1) + (si % IPP) * G::TPI : ptok0 + si * G::TPI;
-      uint32_t vk = voff_k[FP8 ? (i & 1) : (i & 3)], vv = voff_v[FP8 ? ((i >> 1) & 1) : (i & 1)];
+      uint32_t vk = voff_k[k_sel(i)], vv = voff_v[v_sel(i)];
       if (si == i_last && ts > t_last) {  // (also every instruction past i_last: si is clamped)
         uint32_t back = (uint32_t)(ts - t_last) * row_stride;
         vk -= back;
@@ -778,7 +782,7 @@ __global__ __launch_bounds__(NW * 64, SH ? 2 : 1) void paged_decode_mfma_kernel(
         TM(tm_issue)
         wait_stage(u);
         if (SH) {
-          // Own half of tile u has landed; past the barrier so has the partner's, and every wave of the workgroup
+          // Own part of tile u has landed; past the barrier so have the others', and every wave of the workgroup
           // has finished reading tile u-1, whose slot the next fetch overwrites.
           asm volatile("s_barrier" ::: "memory");
         }
@@ -937,21 +941,19 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
 // Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
-// Ring depth of the pair-shared variants, four pairs (eight waves) a compute unit: fp8 4 x 8.25 KiB, 16-bit 2 x 16 KiB a pair.
-template <typename KVT> constexpr int kSharedStages = Geom<KVT>::FP8 ? 4 : 2;
-
 template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB <= 2) ? 8 : 4; }
 
-template <typename QT, typename KVT, int NRB, int NS, int NW, bool SH>
+template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW>
 const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
-  // shared-stage variant: 8 XCDs x (pairs of a group) x ceil(groups / 8), a group being one (partition, kv head); the
-  // pairs of groups past the last exit at once
-  const int grid = SH ? 8 * (n_rg / 2) * ((p.n_parts * p.heads_kv + 7) / 8) : (int)((waves + NW - 1) / NW);
+  constexpr bool SH = SHW > 1;
+  // shared-stage variant: 8 XCDs x (workgroups of a group) x ceil(groups / 8), a group being one (partition, kv head);
+  // the workgroups of groups past the last exit at once
+  const int grid = SH ? 8 * (n_rg / SHW) * ((p.n_parts * p.heads_kv + 7) / 8) : (int)((waves + NW - 1) / NW);
   const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT>::STAGE;
-  if (SH && (n_rg % 2 != 0 || NW != 2)) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
-  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SH>;
+  if (SH && n_rg % SHW != 0) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
+  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SHW>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
   static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
   int dev = 0;
@@ -979,12 +981,17 @@ const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
   constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
   if constexpr (NRB == 2) {
-    // Two or more row groups per kv head would each fetch the same K/V tiles: pair them up on one LDS ring (half the
-    // fetch instructions per wave, one trip through the memory system per tile), the ring twice as deep.
+    // Two or more row groups per kv head would each fetch the same K/V tiles: put 8, 4 or 2 of them on one LDS ring
+    // (a fraction of the fetch instructions per wave, one trip through the memory system per tile).  Eight waves a
+    // compute unit either way; the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
     const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
-    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, kSharedStages<KVT>, 2, true>(p, ws_prefix, skip_combine, s);
+    if constexpr (!Geom<KVT>::FP8) {
+      if (n_rg % 8 == 0) return launch_t4<QT, KVT, NRB, 4, 8, 8>(p, ws_prefix, skip_combine, s);
+    }
+    if (n_rg % 4 == 0) return launch_t4<QT, KVT, NRB, 4, 4, 4>(p, ws_prefix, skip_combine, s);
+    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, Geom<KVT>::FP8 ? 4 : 2, 2, 2>(p, ws_prefix, skip_combine, s);
   }
-  return launch_t4<QT, KVT, NRB, NS, NW, false>(p, ws_prefix, skip_combine, s);
+  return launch_t4<QT, KVT, NRB, NS, NW, 1>(p, ws_prefix, skip_combine, s);
 }
 
 // Row blocks (16 query rows each) per wave.  Above 32 rows an fp8 cache keeps two (its waves hold no accumulation
