@@ -5,8 +5,9 @@
 // the exp2 domain over the paged K/V rows, all query rows that share the kv head served from one read of
 // K/V; partial results merged by log-sum-exp weights.  How it is organised is specific to CDNA4:
 //
-//  * Work unit = one wave.  A wave owns (partition, kv head, block of query rows) and runs on its own: no
-//    workgroup barrier anywhere.  The KV "tile stream" (every 32-token tile of every sequence, in batch
+//  * Work unit = one wave.  A wave owns (partition, kv head, block of query rows) and runs on its own; only when a
+//    kv head has several blocks of query rows do 2, 4 or 8 such waves share their LDS stages and meet at one
+//    barrier per tile (see the kernel's template parameter SHW).  The KV "tile stream" (every 32-token tile of every sequence, in batch
 //    order) is cut into n_parts equal contiguous ranges computed on the device from real_seqlen_kv, so all
 //    compute units get the same number of tiles whatever the length distribution, and nothing is read back
 //    to the host.  A range that covers a whole sequence writes the output directly; a range that starts or
