@@ -247,6 +247,41 @@ def test_multi_token_causal_chunk(kernel_key, fp8, q_len, is_causal):
         torch.testing.assert_close(out[:, i].float(), single(*args).float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("dtype, fp8, tol", [(torch.bfloat16, False, 2e-2), (torch.float16, False, 2e-2), (torch.bfloat16, True, 3e-2),
+                                             (torch.float16, True, 3e-2)])
+@pytest.mark.parametrize(
+    "q_len, heads, heads_kv",
+    [
+        pytest.param(8, 64, 8, id="rows64-ring-of-2"),
+        pytest.param(16, 24, 3, id="rows128-ring-of-4-three-kv-heads"),
+        pytest.param(12, 8, 1, id="rows96-odd-row-groups-one-kv-head"),
+        pytest.param(24, 16, 2, id="rows192-six-row-groups-ring-of-2"),
+        pytest.param(32, 64, 8, id="rows256-ring-of-8-or-4"),
+        pytest.param(40, 16, 2, id="rows320-ten-row-groups"),
+    ],
+)
+def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, heads, heads_kv):
+    """More than 32 query rows per kv head: the row groups of a kv head run as 2, 4 or 8 waves around one LDS ring (or
+    fall back to one wave of four row blocks when their number is odd).  Ragged lengths so that partitions start and
+    end inside sequences, tails shorter than a tile, a sequence shorter than the chunk, NaN in every unaddressed token;
+    head counts that leave the grid with workgroups past the last (partition, kv head)."""
+    require_gfx950()
+    lens = [2100, q_len, q_len + 33, 700, q_len + 31, q_len + 1]
+    case = _ragged_case(len(lens), heads, heads_kv, 128, 64, lens, dtype, q_len=q_len, fp8=fp8, seed=31)
+    op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], 128, 64, is_causal=True)
+    if not _serves(op, "gqa_decode_paged_mfma_kernel", dtype, fp8):
+        pytest.skip("the MFMA kernel does not serve this shape")
+    _force(op, "gqa_decode_paged_mfma_kernel")
+    out = _run_and_compare(op, case, 64, tol, is_causal=True)
+    # and against the other implementation, which shares none of the tiling
+    other = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], 128, 64, is_causal=True)
+    if _serves(other, "gqa_decode_paged_kernel", dtype, fp8):
+        _force(other, "gqa_decode_paged_kernel")
+        dev = [None if t is None else t.to(DEV) for t in case]
+        ref2 = other(*dev[:5]) if case[5] is None else other(*dev)
+        torch.testing.assert_close(out.float(), ref2.float(), atol=tol, rtol=tol)
+
+
 @pytest.mark.parametrize("softcap", [0.0, 30.0])
 def test_closed_forms_on_device(softcap):
     require_gfx950()
