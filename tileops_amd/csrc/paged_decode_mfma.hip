@@ -46,6 +46,11 @@ constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of 
 constexpr int kD = 128;       // head dim served by this kernel
 constexpr int kNumCU = 256;   // MI355X
 constexpr bool kLateIssueFp8 = true;
+
+// Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
+// hold row groups past the last query row, which load nothing, mask everything and store nothing.
+__host__ __device__ constexpr int row_groups(int rows, int nrb) { return (rows + 16 * nrb - 1) / (16 * nrb); }
+__host__ __device__ constexpr int ring_row_groups(int rows, int nrb, int shw) { return (row_groups(rows, nrb) + shw - 1) / shw * shw; }
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT> struct Geom {
@@ -235,7 +240,7 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
   const uint64_t tm_wall0 = wall_clock64();  // constant 100 MHz, common to all XCDs (the cycle counter is per XCD clock)
 #endif
   const int gw = blockIdx.x * NW + wave;
-  const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
+  const int n_rg = ring_row_groups(p.rows, NRB, SHW);
   const int per_part = p.heads_kv * n_rg;
   // integer division runs on the vector ALU; pin the results to scalar registers so that everything derived
   // from them (pool base pointers, LDS bases) is scalar arithmetic
@@ -939,21 +944,19 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
   store(acc0 * inv, acc1 * inv, W > 0.f ? M + log2f(W) : -INFINITY);
 }
 
-// Waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
+// Unshared waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
-template <typename KVT, int NRB> constexpr int waves_per_wg() { return (Geom<KVT>::FP8 && NRB <= 2) ? 8 : 4; }
 
 template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW>
 const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
+  const int n_rg = ring_row_groups(p.rows, NRB, SHW);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
   constexpr bool SH = SHW > 1;
   // shared-stage variant: 8 XCDs x (workgroups of a group) x ceil(groups / 8), a group being one (partition, kv head);
   // the workgroups of groups past the last exit at once
   const int grid = SH ? 8 * (n_rg / SHW) * ((p.n_parts * p.heads_kv + 7) / 8) : (int)((waves + NW - 1) / NW);
   const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT>::STAGE;
-  if (SH && n_rg % SHW != 0) return "MFMA kernel: shared-stage variant launched on a shape it does not fit";
   auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SHW>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
   static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
@@ -977,38 +980,34 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
-template <typename QT, typename KVT, int NRB>
-const char* launch_t3(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  // two stages per wave; the fp8 multi-row-block variants have LDS to spare (one wave per SIMD) and take three
-  constexpr int NS = (Geom<KVT>::FP8 && NRB > 2) ? 3 : 2, NW = waves_per_wg<KVT, NRB>();
-  if constexpr (NRB == 2) {
-    // Two or more row groups per kv head would each fetch the same K/V tiles: put 8, 4 or 2 of them on one LDS ring
-    // (a fraction of the fetch instructions per wave, one trip through the memory system per tile).  Eight waves a
-    // compute unit either way; the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
-    const int n_rg = (p.rows + 16 * NRB - 1) / (16 * NRB);
-    if constexpr (!Geom<KVT>::FP8) {
-      if (n_rg % 8 == 0) return launch_t4<QT, KVT, NRB, 4, 8, 8>(p, ws_prefix, skip_combine, s);
-    }
-    if (n_rg % 4 == 0) return launch_t4<QT, KVT, NRB, 4, 4, 4>(p, ws_prefix, skip_combine, s);
-    if (n_rg % 2 == 0) return launch_t4<QT, KVT, NRB, Geom<KVT>::FP8 ? 4 : 2, 2, 2>(p, ws_prefix, skip_combine, s);
-  }
-  return launch_t4<QT, KVT, NRB, NS, NW, 1>(p, ws_prefix, skip_combine, s);
-}
+// Row blocks (16 query rows each) per wave: one up to 16 rows per kv head, else two.
+int row_blocks_for(int rows) { return rows <= 16 ? 1 : 2; }
 
-// Row blocks (16 query rows each) per wave.  Above 32 rows an fp8 cache keeps two (its waves hold no accumulation
-// registers to spare); a 16-bit cache takes two when the row groups pair up on shared stages, else four.
-int row_blocks_for(int rows, bool fp8) {
-  if (rows <= 16) return 1;
-  if (rows <= 32 || fp8) return 2;
-  return ((rows + 31) / 32) % 2 == 0 ? 2 : 4;
+// Waves per LDS ring.  Up to 32 rows per kv head there is one row group and every wave has its own ring.  Beyond, the
+// 32-row groups of a kv head would each fetch the same K/V tiles: 8, 4 or 2 of them share one ring (a fraction of the
+// fetch instructions per wave, one trip through the memory system per tile); an odd count is rounded up by one idle
+// row group.  Eight waves a compute unit either way (accumulators of two row blocks fit ordinary vector registers);
+// the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
+int ring_waves_for(int rows, bool fp8) {
+  const int n = row_groups(rows, 2);
+  if (rows <= 32) return 1;
+  const int even = (n + 1) / 2 * 2;
+  if (even % 8 == 0 && !fp8) return 8;
+  if (even % 4 == 0) return 4;
+  return 2;
 }
 
 template <typename QT, typename KVT>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  switch (row_blocks_for(p.rows, Geom<KVT>::FP8)) {
-    case 1: return launch_t3<QT, KVT, 1>(p, ws_prefix, skip_combine, s);
-    case 2: return launch_t3<QT, KVT, 2>(p, ws_prefix, skip_combine, s);
-    default: return launch_t3<QT, KVT, 4>(p, ws_prefix, skip_combine, s);
+  constexpr bool FP8 = Geom<KVT>::FP8;
+  if (row_blocks_for(p.rows) == 1) return launch_t4<QT, KVT, 1, 2, FP8 ? 8 : 4, 1>(p, ws_prefix, skip_combine, s);
+  switch (ring_waves_for(p.rows, FP8)) {
+    case 1: return launch_t4<QT, KVT, 2, 2, FP8 ? 8 : 4, 1>(p, ws_prefix, skip_combine, s);
+    case 2: return launch_t4<QT, KVT, 2, FP8 ? 4 : 2, 2, 2>(p, ws_prefix, skip_combine, s);
+    case 4: return launch_t4<QT, KVT, 2, 4, 4, 4>(p, ws_prefix, skip_combine, s);
+    default:
+      if constexpr (!FP8) return launch_t4<QT, KVT, 2, 4, 8, 8>(p, ws_prefix, skip_combine, s);
+      return "MFMA kernel: no ring of eight waves for an fp8 cache";
   }
 }
 
@@ -1027,13 +1026,12 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 // Number of equal ranges the tile stream is cut into: one wave per (range, kv head, row group), sized so
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
 int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
-  const int nrb = row_blocks_for(rows, kv_dtype == MI355_DT_FP8_E4M3FN);
-  const int n_rg = (rows + 16 * nrb - 1) / (16 * nrb);
-  // resident waves per CU: eight for the fp8 single-row-block kernel (LDS-limited, ~160 VGPRs), otherwise four
-  // (LDS-limited with a 16-bit cache, register-limited -- one wave per SIMD -- with more than one row block)
-  // -- and eight again for wave pairs on shared stages, which keep their accumulators in ordinary vector registers
-  const bool shared = nrb == 2 && n_rg % 2 == 0;
-  const int waves_per_cu = ((kv_dtype == MI355_DT_FP8_E4M3FN && nrb <= 2) || shared) ? 8 : 4;
+  const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
+  const int nrb = row_blocks_for(rows), shw = ring_waves_for(rows, fp8);
+  const int n_rg = ring_row_groups(rows, nrb, shw);
+  // resident waves per CU: eight with an fp8 cache (LDS-limited) and for shared rings (accumulators in ordinary
+  // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
+  const int waves_per_cu = (fp8 || shw > 1) ? 8 : 4;
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;

@@ -30,13 +30,19 @@ TIMER_LIB = Path(build_mod.LIB_PATH).with_name("libmi355_tileops_phase_timers.so
 NAMES = ("issue", "wait", "compute", "segment", "prologue", "total")
 
 
-def _row_blocks(rows: int, fp8: bool) -> int:
+def _row_blocks(rows: int) -> int:
     """Row blocks per wave the launcher picks (csrc/paged_decode_mfma.hip: row_blocks_for)."""
-    if rows <= 16:
+    return 1 if rows <= 16 else 2
+
+
+def _ring_waves(rows: int, fp8: bool) -> int:
+    """Waves per shared LDS ring (csrc/paged_decode_mfma.hip: ring_waves_for)."""
+    if rows <= 32:
         return 1
-    if rows <= 32 or fp8:
-        return 2
-    return 2 if ((rows + 31) // 32) % 2 == 0 else 4
+    even = ((rows + 31) // 32 + 1) // 2 * 2
+    if even % 8 == 0 and not fp8:
+        return 8
+    return 4 if even % 4 == 0 else 2
 
 
 def run(name: str, hot: bool = False) -> None:
@@ -50,13 +56,12 @@ def run(name: str, hot: bool = False) -> None:
                                                 inp.block_table.shape[1], inp.q.dtype, inp.k.dtype, 0, native.KERNEL_MFMA)
     fp8 = inp.k.dtype == FP8
     rows = cfg.q_len * (cfg.heads // cfg.heads_kv)
-    nrb = _row_blocks(rows, fp8)
-    n_rg = (rows + 16 * nrb - 1) // (16 * nrb)
+    nrb, shw = _row_blocks(rows), _ring_waves(rows, fp8)
+    n_rg = ((rows + 16 * nrb - 1) // (16 * nrb) + shw - 1) // shw * shw  # whole rings
     waves = nparts * cfg.heads_kv * n_rg
-    shared = nrb == 2 and n_rg % 2 == 0  # wave pairs sharing an LDS ring (csrc/paged_decode_mfma.hip: launch_t3)
-    nw = 2 if shared else (8 if (fp8 and nrb <= 2) else 4)  # waves per workgroup
-    if shared:
-        waves = 2 * 8 * (n_rg // 2) * ((nparts * cfg.heads_kv + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
+    nw = shw if shw > 1 else (8 if fp8 else 4)  # waves per workgroup
+    if shw > 1:
+        waves = shw * 8 * (n_rg // shw) * ((nparts * cfg.heads_kv + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
     ws = torch.zeros(nbytes + waves * 32 + 4096, dtype=torch.uint8, device=dev)
     flush_w = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     flush_r = torch.ones(128 << 20, dtype=torch.int32, device=dev)
