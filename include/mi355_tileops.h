@@ -165,6 +165,34 @@ int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new,
                             float sm_scale, float softcap, int causal, int kernel, void* hip_stream);
 
 /*
+ * The same prefill chunk with rotary position embedding fused in (GPT-NeoX halves), 16-bit cache only.  Replaces
+ * GQAPrefillPagedWithKVCacheRopeFwdKernel.forward and its two TileLang kernels
+ * (src/tileops/kernels/attention/gqa_fwd.py:1464-1582 append, :1660-1917 attention, :2020-2090 class); op side
+ * src/tileops/ops/attention/gqa.py:787-823, :891-895, :1048-1065, :1113-1143.
+ * Query and new key rows of token t of sequence b are rotated at logical position cache_seqlens[b] + (t - cu_q[b]):
+ *   y[d] = x[d]*cos[pos][d % half] + r*sin[pos][d % half],  half = rotary_dim / 2,
+ *   r = -x[d + half] for d < half, +x[d - half] for half <= d < rotary_dim;  y[d] = x[d] for d >= rotary_dim
+ * (gqa_fwd.py:1521-1535, :1755-1768), products in fp32, rounded once to q_dtype.  The rotated keys go into the pages
+ * (values are copied), the rotated queries into the workspace, and attention runs as in mi355_gqa_prefill_paged.
+ *   cos_table,
+ *   sin_table      [max_position, rotary_dim / 2] q_dtype (src/tileops/ops/rope.py:97-120)
+ *   rotary_dim     even, 0 < rotary_dim <= dim
+ *   max_position   rows of the tables; the caller guarantees cache_seqlens[b] + q_len_b <= max_position
+ *                  (gqa.py:1032-1036); positions beyond are clamped to the last row rather than read out of bounds
+ * q, k_new and v_new are not modified.
+ */
+int mi355_gqa_prefill_paged_rope_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
+                                           int page_size, int64_t max_pages_per_req, int q_dtype, int kernel,
+                                           size_t* workspace_bytes);
+int mi355_gqa_prefill_paged_rope(const void* q, const void* k_new, const void* v_new, void* k_pages, void* v_pages,
+                                 const void* cos_table, const void* sin_table, const int32_t* cu_seqlens_q,
+                                 const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,
+                                 void* workspace, size_t workspace_bytes, int batch, int max_seqlen_q, int64_t total_q,
+                                 int heads, int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype,
+                                 int rotary_dim, int64_t max_position, float sm_scale, float softcap, int causal, int kernel,
+                                 void* hip_stream);
+
+/*
  * Index-probe: materialise the logical KV rows a decode call would read, with the same device page
  * arithmetic the attention kernels use.  dense_out [batch, max_len, heads_kv * dim] elem_bytes-wide
  * elements; rows t >= seqlens[b] are left untouched.  Lets a test compare the gather bit-for-bit with

@@ -18,6 +18,12 @@ Parity status of each function (how it is pinned, without importing the referenc
 * ``ref_gqa_prefill_paged``     pinned against SDPA per sequence (explicit boolean mask), against "row i of a chunk ==
                                 single-token decode over old tokens + chunk[:i+1]" through the pinned decode oracle,
                                 and, for the append, against a per-token loop over ``physical_pos`` and torch's fp8 cast.
+* ``rope_tables`` / ``apply_neox_rope`` / ``ref_gqa_prefill_paged_rope``
+                                pinned by what the mathematics fixes: position 0 is the identity; each (d, d+half) pair is
+                                rotated by exactly ``pos * base**(-i/half)`` (checked against complex multiplication in
+                                float64); pair norms are preserved; ``<rope(q, m), rope(k, n)>`` depends on ``m - n`` only;
+                                dimensions past ``rotary_dim`` pass through bit for bit; the fused op equals "rotate, then
+                                the pinned plain prefill oracle".
 
 The exact floating-point bits of the reference's TileLang-generated CUDA kernels are not reproducible here
 (TileLang is absent); the reference itself defines correctness against this torch program within tolerance.
@@ -321,3 +327,66 @@ def ref_gqa_prefill_paged(
                 k_after[pos] = k_new[q0 + i]
                 v_after[pos] = v_new[q0 + i]
     return out, k_after, v_after
+
+
+def rope_tables(rotary_dim: int, max_position: int, base: float = 10000.0, dtype: torch.dtype = torch.float32) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos/sin ``[max_position, rotary_dim // 2]``: ``angle[p, i] = p * base**(-i / half)`` evaluated in fp32, then cast
+    to *dtype*.  src/tileops/ops/rope.py:97-120 (``base_freqs``)."""
+    half = rotary_dim // 2
+    freqs = 1.0 / (base ** (torch.arange(0, half, dtype=torch.float32) / half))
+    angles = torch.outer(torch.arange(max_position, dtype=torch.float32), freqs)
+    return torch.cos(angles).to(dtype), torch.sin(angles).to(dtype)
+
+
+def apply_neox_rope(x: torch.Tensor, positions: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor,
+                    rotary_dim: Optional[int] = None) -> torch.Tensor:
+    """GPT-NeoX rotary embedding of packed rows ``x [T, heads, D]`` at ``positions [T]``:
+    ``y[d] = x[d]*c + r*s`` with ``c, s = table[pos, d % half]``, ``r = -x[d + half]`` for ``d < half``, ``+x[d - half]``
+    for ``half <= d < rotary_dim``; dimensions from ``rotary_dim`` on pass through
+    (src/tileops/kernels/rope.py:228-246; the fused prefill kernels: kernels/attention/gqa_fwd.py:1521-1535, :1755-1768).
+    The reference evaluates the expression on 16-bit operands inside TileLang; here the products are formed in fp32 from
+    the same 16-bit operands (tables included) and rounded once to ``x.dtype`` -- at most an ulp or two apart."""
+    D = x.shape[-1]
+    rotary_dim = D if rotary_dim is None else rotary_dim
+    half = rotary_dim // 2
+    pos = positions.long()
+    work = torch.float64 if x.dtype == torch.float64 else torch.float32
+    c = cos_table[pos].to(work)[:, None, :]  # [T, 1, half]
+    s = sin_table[pos].to(work)[:, None, :]
+    xf = x.to(work)
+    lo, hi = xf[..., :half], xf[..., half:rotary_dim]
+    y = xf.clone()
+    y[..., :half] = lo * c - hi * s
+    y[..., half:rotary_dim] = hi * c + lo * s
+    return y.to(x.dtype)
+
+
+def ref_gqa_prefill_paged_rope(
+    q: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cache_seqlens: torch.Tensor,
+    block_table: torch.Tensor,
+    cos_table: torch.Tensor,
+    sin_table: torch.Tensor,
+    *,
+    page_size: int,
+    rotary_dim: Optional[int] = None,
+    is_causal: bool = True,
+    sm_scale: Optional[float] = None,
+    softcap: float = 0.0,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The prefill chunk with fused rotary embedding, as the reference's test builds its expectation
+    (tests/ops/attention/test_gqa_prefill_paged.py:485-600): rotate ``q`` and ``k_new`` at positions
+    ``cache_seqlens[b] + i`` (the cache already holds rotated keys), then the plain chunk semantics on the rotated
+    tensors; the pages receive the rotated keys and the untouched values."""
+    positions = torch.cat([torch.arange(int(cache_seqlens[b]), int(cache_seqlens[b]) + int(cu_seqlens_q[b + 1]) - int(cu_seqlens_q[b]))
+                           for b in range(cache_seqlens.shape[0])]).to(torch.int32)
+    q_rot = apply_neox_rope(q, positions, cos_table, sin_table, rotary_dim)
+    k_rot = apply_neox_rope(k_new, positions, cos_table, sin_table, rotary_dim)
+    one = torch.ones(1, dtype=torch.float32)
+    return ref_gqa_prefill_paged(q_rot, k_rot, v_new, k_pages, v_pages, one, one, cu_seqlens_q, cache_seqlens, block_table,
+                                 page_size=page_size, is_causal=is_causal, sm_scale=sm_scale, softcap=softcap)

@@ -14,7 +14,8 @@ import torch
 import torch.nn.functional as F
 
 from oracle.paged_gqa_decode_ref import (
-    physical_pos, quantize_per_tensor, ref_gqa_prefill_paged, ref_paged_gqa_decode,
+    apply_neox_rope, physical_pos, quantize_per_tensor, ref_gqa_prefill_paged, ref_gqa_prefill_paged_rope, ref_paged_gqa_decode,
+    rope_tables,
 )
 from tests.conftest import require_gfx950
 from tileops_amd import native
@@ -109,6 +110,55 @@ def test_oracle_append_touches_exactly_the_chunk_positions_and_quantises_like_a_
         assert torch.equal(v_after[~touched].view(torch.uint8), v_pages[~touched].view(torch.uint8))
 
 
+def test_oracle_rope_is_a_rotation_of_each_pair_by_position_times_frequency():
+    """Pins ``rope_tables`` / ``apply_neox_rope`` by what the mathematics fixes (float64 tables, so that only the formula
+    is on trial): position 0 is the identity; the pair (x[i], x[i + half]) read as a complex number is multiplied by
+    exp(j * pos * base**(-i/half)); pair norms are preserved; dimensions from rotary_dim on pass through bit for bit;
+    and <rope(q, m), rope(k, n)> depends on m - n only."""
+    g = torch.Generator().manual_seed(5)
+    D, rd, base, P = 64, 32, 10000.0, 300
+    half = rd // 2
+    cos, sin = rope_tables(rd, P, base, torch.float64)
+    assert cos.shape == (P, half) and sin.shape == (P, half)
+    x = torch.randn(7, 3, D, generator=g, dtype=torch.float64)
+    pos = torch.tensor([0, 1, 2, 17, 100, 255, 299], dtype=torch.int32)
+    y = apply_neox_rope(x, pos, cos, sin, rd)
+    assert torch.equal(y[0], x[0])                                  # position 0
+    assert torch.equal(y[..., rd:], x[..., rd:])                    # the tail is untouched
+    zx = torch.complex(x[..., :half], x[..., half:rd])
+    zy = torch.complex(y[..., :half], y[..., half:rd])
+    freqs = base ** (-torch.arange(half, dtype=torch.float64) / half)
+    expect = zx * torch.exp(1j * pos.double()[:, None, None] * freqs)
+    # the tables come from fp32 angles (as the reference builds them): |angle error| <= ~300 * 2^-24
+    torch.testing.assert_close(zy, expect, atol=5e-5, rtol=0)
+    torch.testing.assert_close(zy.abs(), zx.abs(), atol=0, rtol=5e-7)   # a rotation, up to cos^2 + sin^2 of fp32 table entries
+    # relative-position property (on a full rotary_dim, with one row at two position pairs of equal distance)
+    cos2, sin2 = rope_tables(D, P, base, torch.float64)
+    qv, kv = torch.randn(1, 1, D, generator=g, dtype=torch.float64), torch.randn(1, 1, D, generator=g, dtype=torch.float64)
+    def dot(m, n):
+        a = apply_neox_rope(qv, torch.tensor([m]), cos2, sin2)
+        b = apply_neox_rope(kv, torch.tensor([n]), cos2, sin2)
+        return float((a * b).sum())
+    assert abs(dot(40, 10) - dot(130, 100)) < 2e-4 and abs(dot(40, 10) - dot(41, 10)) > 1e-3
+
+
+def test_oracle_fused_rope_prefill_is_rotate_then_plain_prefill_and_tables_round_like_the_reference():
+    q_lens, old_lens, dtype = [5, 3], [7, 70], torch.float16
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = _case(q_lens, old_lens, 4, 2, 64, dtype, seed=9)
+    cos, sin = rope_tables(32, 128, 10000.0, dtype)
+    assert cos.dtype == dtype and float(cos[0].min()) == 1.0 and float(sin[0].abs().max()) == 0.0
+    out, k_after, v_after = ref_gqa_prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cu, cache, table, cos, sin,
+                                                       page_size=64, rotary_dim=32)
+    positions = torch.tensor([7, 8, 9, 10, 11, 70, 71, 72], dtype=torch.int32)
+    k_rot = apply_neox_rope(k_new, positions, cos, sin, 32)
+    for t, (b, i) in enumerate([(0, 0), (0, 1), (0, 2), (0, 3), (0, 4), (1, 0), (1, 1), (1, 2)]):
+        pos = physical_pos(table, b, old_lens[b] + i, 64)
+        assert torch.equal(k_after[pos], k_rot[t]) and torch.equal(v_after[pos], v_new[t])
+    plain, _, _ = ref_gqa_prefill_paged(apply_neox_rope(q, positions, cos, sin, 32), k_rot, v_new, k_pages, v_pages, ks, vs, cu,
+                                        cache, table, page_size=64)
+    assert torch.equal(out, plain)
+
+
 def test_roofline_formula_by_hand():
     """src/tileops/perf/formulas.py:567-587 on the reference's llama-8b row: 8 x (512 new, 4096 old), fp16."""
     flops, nbytes = gqa_prefill_paged_with_kv_cache_fwd_roofline(
@@ -132,6 +182,8 @@ def test_op_constructs_without_device_and_validates_like_the_reference():
         PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, fuse_rope=True)
     with pytest.raises(ValueError, match="rotary_dim requires fuse_rope=True"):
         PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, rotary_dim=32)
+    with pytest.raises(ValueError, match="rotary_dim must be"):
+        PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, fuse_rope=True, max_position=512, rotary_dim=31)
     with pytest.raises(ValueError, match="fuse_rope is not supported with FP8 paged KV cache yet"):
         PrefillOp(batch=1, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, fuse_rope=True, max_position=512, cache_dtype=FP8)
     with pytest.raises(NotImplementedError):
@@ -253,3 +305,92 @@ def test_llama_shape_chunks_of_hundreds_of_rows_against_long_prefixes(fp8):
     case = _case(q_lens, old_lens, 32, 8, 128, torch.float16, fp8=fp8, page=64, max_pages=72, seed=21)
     op = PrefillOp(batch=2, heads=32, heads_kv=8, max_pages_per_req=72, page_size=64, dim=128, cache_dtype=FP8 if fp8 else None)
     _run(op, case, 64, torch.float16, fp8=fp8)
+
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "rotary_dim, is_causal, softcap",
+    [pytest.param(None, True, None, id="full-causal"), pytest.param(32, True, None, id="partial-causal"),
+     pytest.param(32, False, None, id="partial-noncausal"), pytest.param(32, True, 2.0, id="partial-causal-softcap"),
+     pytest.param(30, True, None, id="odd-number-of-pairs")],
+)
+def test_gqa_prefill_paged_with_kv_cache_fused_rope(rotary_dim, is_causal, softcap):
+    """The reference's fused-RoPE case (tests/ops/attention/test_gqa_prefill_paged.py:476-600): raw q / k_new in, the
+    cache holds rotated old keys; output against "rotate, then plain prefill", appended keys equal the rotated new
+    keys, values are copied, old tokens and the inputs are untouched."""
+    require_gfx950()
+    q_lens, old_lens, heads, heads_kv, dim, dtype = [48, 33], [67, 100], 8, 2, 64, torch.float16
+    max_position = max(o + n for o, n in zip(old_lens, q_lens)) + 1
+    _fused_rope_case(q_lens, old_lens, heads, heads_kv, dim, dtype, rotary_dim, max_position, is_causal, softcap, atol=5e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype, atol", [(torch.bfloat16, 3e-2), (torch.float16, 5e-3)])
+@pytest.mark.parametrize("kernel", ["auto", "generic"])
+def test_fused_rope_head_dim_128_long_positions_empty_chunk_and_empty_cache(dtype, atol, kernel):
+    """Head dim 128 (MFMA path), positions in the thousands (where bf16 tables are coarse), a sequence with nothing
+    cached, one with an empty chunk, a chunk that crosses a page boundary."""
+    require_gfx950()
+    q_lens, old_lens = [70, 0, 9, 130], [0, 300, 1999, 62]
+    _fused_rope_case(q_lens, old_lens, 16, 4, 128, dtype, 64, 2100, True, None, atol=atol, max_pages=33,
+                     config={"kernel": native.KERNEL_GENERIC} if kernel == "generic" else None)
+
+
+def _fused_rope_case(q_lens, old_lens, heads, heads_kv, dim, dtype, rotary_dim, max_position, is_causal, softcap, *, atol,
+                     max_pages=8, config=None):
+    g = torch.Generator().manual_seed(41)
+    batch, total_q, page = len(q_lens), sum(q_lens), 64
+    rd = dim if rotary_dim is None else rotary_dim
+    op = PrefillOp(batch=batch, heads=heads, heads_kv=heads_kv, max_pages_per_req=max_pages, page_size=page, dim=dim,
+                   is_causal=is_causal, softcap=softcap, fuse_rope=True, max_position=max_position, rotary_dim=rotary_dim)
+    # The op builds its tables on the device, like the reference (ops/attention/gqa.py:1048-1065); device and host
+    # cos/sin may disagree in the last fp32 bit, hence now and then in the last 16-bit one.  The tables are pinned
+    # against the oracle's to that one ulp, and the rotation is then checked with the very tables the kernel reads.
+    cos, sin = (t.cpu() for t in op._rope_tables(torch.device(DEV, 0), dtype))
+    cos_ref, sin_ref = rope_tables(rd, max_position, 10000.0, dtype)
+    one_ulp = torch.finfo(dtype).eps
+    torch.testing.assert_close(cos.float(), cos_ref.float(), atol=one_ulp, rtol=0)
+    torch.testing.assert_close(sin.float(), sin_ref.float(), atol=one_ulp, rtol=0)
+    assert float((cos != cos_ref).float().mean()) < 0.05 and float((sin != sin_ref).float().mean()) < 0.05
+    table = _block_table(batch, max_pages)
+    cu = torch.tensor([0, *accumulate(q_lens)], dtype=torch.int32)
+    cache = torch.tensor(old_lens, dtype=torch.int32)
+    q = torch.randn(total_q, heads, dim, generator=g).to(dtype)
+    k_new = torch.randn(total_q, heads_kv, dim, generator=g).to(dtype)
+    v_new = torch.randn(total_q, heads_kv, dim, generator=g).to(dtype)
+    k_pages = torch.zeros(batch * max_pages * page, heads_kv, dim, dtype=dtype)
+    v_pages = torch.zeros_like(k_pages)
+    for b, old in enumerate(old_lens):
+        if old == 0:
+            continue
+        ko = apply_neox_rope(torch.randn(old, heads_kv, dim, generator=g).to(dtype), torch.arange(old, dtype=torch.int32), cos, sin, rd)
+        vo = torch.randn(old, heads_kv, dim, generator=g).to(dtype)
+        idx = torch.tensor([physical_pos(table, b, t, page) for t in range(old)])
+        k_pages[idx], v_pages[idx] = ko, vo
+    ref, k_after, v_after = ref_gqa_prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cu, cache, table, cos, sin, page_size=page,
+                                                       rotary_dim=rd, is_causal=is_causal, softcap=softcap or 0.0)
+    if config is not None:
+        key = "gqa_prefill_paged_with_kv_cache_rope_fwd_kernel"
+        base = op.kernel_map[key]
+        op.kernel_map = dict(op.kernel_map)
+        op.kernel_map[key] = type("Forced", (base,), {"default_config": property(lambda self: dict(config))})
+    dev = [t.to(DEV) for t in (q, k_new, v_new, k_pages, v_pages)]
+    one = torch.ones(1, dtype=torch.float32, device=DEV)
+    q_before, k_before = dev[0].clone(), dev[1].clone()
+    out = op(*dev, one, one.clone(), cu.to(DEV), cache.to(DEV), table.to(DEV), max(q_lens))
+    torch.cuda.synchronize()
+    assert torch.equal(dev[0], q_before) and torch.equal(dev[1], k_before)          # inputs are not rotated in place
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=atol, rtol=1e-2)
+    # appended keys: the rotated chunk.  Kernel and oracle both evaluate x*c + r*s in fp32 on the same 16-bit operands and
+    # round once, but not with the same fp32 roundings (fused multiply-add or not), so they may differ by one 16-bit ulp of
+    # the result plus, where the two products cancel, a few fp32 ulps of the operands (|x| < 5 here).  Values are copied;
+    # every other row of the pool is as before.
+    assert torch.equal(dev[4].cpu(), v_after)
+    k_dev = dev[3].cpu()
+    torch.testing.assert_close(k_dev.float(), k_after.float(), atol=2e-6, rtol=torch.finfo(dtype).eps)
+    touched = torch.zeros(k_pages.shape[0], dtype=torch.bool)
+    for b, (n, old) in enumerate(zip(q_lens, old_lens)):
+        for i in range(n):
+            touched[physical_pos(table, b, old + i, page)] = True
+    assert torch.equal(k_dev[~touched], k_pages[~touched])

@@ -361,6 +361,66 @@ int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new,
   return MI355_OK;
 }
 
+int mi355_gqa_prefill_paged_rope_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
+                                           int page_size, int64_t max_pages_per_req, int q_dtype, int kernel,
+                                           size_t* workspace_bytes) {
+  size_t base = 0;
+  int rc = mi355_gqa_prefill_paged_workspace(batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, max_pages_per_req,
+                                             q_dtype, q_dtype, kernel, &base);
+  if (rc) return rc;
+  // the rotated queries follow the attention workspace
+  if (workspace_bytes) *workspace_bytes = align256(base) + align256((size_t)total_q * heads * dim * 2);
+  return MI355_OK;
+}
+
+int mi355_gqa_prefill_paged_rope(const void* q, const void* k_new, const void* v_new, void* k_pages, void* v_pages,
+                                 const void* cos_table, const void* sin_table, const int32_t* cu_seqlens_q,
+                                 const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,
+                                 void* workspace, size_t workspace_bytes, int batch, int max_seqlen_q, int64_t total_q,
+                                 int heads, int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype,
+                                 int rotary_dim, int64_t max_position, float sm_scale, float softcap, int causal, int kernel,
+                                 void* hip_stream) {
+  int rc = check_shape(batch, max_seqlen_q, heads, heads_kv, dim, page_size, q_dtype, q_dtype);
+  if (rc) return rc;
+  if (rotary_dim <= 0 || rotary_dim % 2 != 0 || rotary_dim > dim)
+    return fail(MI355_EINVAL, "rotary_dim (%d) must be positive, even, and <= dim (%d)", rotary_dim, dim);
+  if (max_position <= 0) return fail(MI355_EINVAL, "max_position must be positive");
+  if (batch == 0 || total_q == 0) return MI355_OK;
+  if (total_q < 0) return fail(MI355_EINVAL, "total_q must be non-negative");
+  if (!q || !k_new || !v_new || !k_pages || !v_pages || !cos_table || !sin_table || !cu_seqlens_q || !cache_seqlens ||
+      !block_table || !out)
+    return fail(MI355_EINVAL, "q, k_new, v_new, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q, cache_seqlens, block_table and out must be non-null");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens, page_size);
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (((uintptr_t)q | (uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)k_pages | (uintptr_t)v_pages | (uintptr_t)cos_table |
+       (uintptr_t)sin_table) & 15)
+    return fail(MI355_EINVAL, "q, k_new, v_new, k_pages, v_pages, cos_table and sin_table must be 16-byte aligned");
+  size_t base = 0, need = 0;
+  rc = mi355_gqa_prefill_paged_workspace(batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype,
+                                         q_dtype, kernel, &base);
+  if (rc) return rc;
+  rc = mi355_gqa_prefill_paged_rope_workspace(batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, bt_row_stride,
+                                              q_dtype, kernel, &need);
+  if (rc) return rc;
+  if (!workspace) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got null", need);
+  if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
+  void* q_rot = (char*)workspace + align256(base);
+  const char* err = launch_rope_append_chunk(q, k_new, v_new, q_rot, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q,
+                                             cache_seqlens, block_table, bt_row_stride, batch, total_q, heads, heads_kv, dim,
+                                             rotary_dim, max_position, page_size, n_phys_tokens / page_size, q_dtype,
+                                             (hipStream_t)hip_stream);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  // the rotated chunk is in the pages now: one pass over (old + new) tokens with the rotated queries
+  Extras ex;
+  ex.cu_q = cu_seqlens_q;
+  ex.len_excludes_new = 1;
+  return run_decode(q_rot, k_pages, v_pages, nullptr, nullptr, cache_seqlens, block_table, bt_row_stride, 0, 0, out, workspace,
+                    align256(base), batch, max_seqlen_q, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype, q_dtype,
+                    sm_scale, softcap, causal, 0, kernel, hip_stream, ex);
+}
+
 int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
                        void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size, int64_t n_phys_tokens,
                        void* hip_stream) {

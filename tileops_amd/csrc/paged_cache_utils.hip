@@ -156,6 +156,125 @@ const char* launch_kv_append_chunk(const void* k_new, const void* v_new, void* k
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
+// Rotary position embedding (GPT-NeoX halves) fused with the chunk append, 16-bit cache: for token t of sequence b at
+// logical position pos = cache_seqlens[b] + (t - cu_q[b]),
+//   y[d] = x[d]*cos[pos][d % half] + r*sin[pos][d % half],  r = -x[d + half] (d < half), +x[d - half] (half <= d < rotary_dim),
+//   y[d] = x[d] for d >= rotary_dim,
+// applied to every query head (written to q_rot) and every key head (written into the pages); V is copied
+// (src/tileops/kernels/attention/gqa_fwd.py:1505-1578 for K/V, :1755-1768 for Q; tables [max_position, half] in the
+// element type, src/tileops/ops/rope.py:97-120).  The products are formed in fp32 from the 16-bit operands and rounded
+// once.  One workgroup per token.
+template <typename XT>
+__device__ __forceinline__ float elem_to_f32(uint16_t bits) {
+  uint32_t raw[1] = {bits};
+  float out[2];
+  Unpack<XT, 2>::run(raw, out);
+  return out[0];
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_new,
+                                                                const uint16_t* __restrict__ v_new, uint16_t* __restrict__ q_rot,
+                                                                uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages,
+                                                                const uint16_t* __restrict__ cos_table, const uint16_t* __restrict__ sin_table,
+                                                                const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
+                                                                const int32_t* __restrict__ block_table, int64_t bt_row_stride, int batch,
+                                                                int heads, int heads_kv, int dim, int rotary_dim, int64_t max_position,
+                                                                int page_size, int64_t n_pages) {
+  const int64_t t = blockIdx.x;
+  int lo = 0, hi = batch;  // the sequence with cu_q[b] <= t < cu_q[b+1] (empty chunks are skipped by the search)
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int b = lo;
+  if (t >= cu_q[b + 1]) return;
+  const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
+  const int64_t tpos = pos < max_position ? pos : max_position - 1;  // the caller checks positions; never read past the tables
+  const int half = rotary_dim >> 1;
+  const uint16_t* cs = cos_table + tpos * half;
+  const uint16_t* sn = sin_table + tpos * half;
+  auto rotate = [&](const uint16_t* x, int d) -> uint16_t {
+    if (d >= rotary_dim) return x[d];
+    const int f = d < half ? d : d - half;
+    const float c = elem_to_f32<XT>(cs[f]), sv = elem_to_f32<XT>(sn[f]), val = elem_to_f32<XT>(x[d]);
+    const float r = d < half ? -elem_to_f32<XT>(x[d + half]) : elem_to_f32<XT>(x[d - half]);
+    return f32_to_elem_bits<XT>(val * c + r * sv);
+  };
+  const int64_t q_elems = (int64_t)heads * dim, kv_elems = (int64_t)heads_kv * dim;
+  const uint16_t* qs = q + t * q_elems;
+  uint16_t* qd = q_rot + t * q_elems;
+  const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages);
+  const uint16_t* ks = k_new + t * kv_elems;
+  const uint16_t* vs = v_new + t * kv_elems;
+  uint16_t* kd = k_pages + phys * kv_elems;
+  uint16_t* vd = v_pages + phys * kv_elems;
+  if ((half & 1) == 0) {
+    // two neighbouring pairs per work item, everything in 4-byte accesses: items [0, half/2) of a head rotate
+    // (d, d+1, d+half, d+half+1), the rest copy the dimensions past rotary_dim two at a time
+    const int rot_items = half >> 1;
+    auto head_item = [&](const uint16_t* x, uint16_t* y, int it) {
+      if (it >= rot_items) {
+        const int d = rotary_dim + 2 * (it - rot_items);
+        *(uint32_t*)(y + d) = *(const uint32_t*)(x + d);
+        return;
+      }
+      const int d = 2 * it;
+      uint32_t lo_raw[1] = {*(const uint32_t*)(x + d)}, hi_raw[1] = {*(const uint32_t*)(x + d + half)};
+      uint32_t c_raw[1] = {*(const uint32_t*)(cs + d)}, s_raw[1] = {*(const uint32_t*)(sn + d)};
+      float lo[2], hi[2], c[2], sv[2];
+      Unpack<XT, 2>::run(lo_raw, lo);
+      Unpack<XT, 2>::run(hi_raw, hi);
+      Unpack<XT, 2>::run(c_raw, c);
+      Unpack<XT, 2>::run(s_raw, sv);
+      const uint32_t o_lo = (uint32_t)f32_to_elem_bits<XT>(lo[0] * c[0] + (-hi[0]) * sv[0]) |
+                            ((uint32_t)f32_to_elem_bits<XT>(lo[1] * c[1] + (-hi[1]) * sv[1]) << 16);
+      const uint32_t o_hi = (uint32_t)f32_to_elem_bits<XT>(hi[0] * c[0] + lo[0] * sv[0]) |
+                            ((uint32_t)f32_to_elem_bits<XT>(hi[1] * c[1] + lo[1] * sv[1]) << 16);
+      *(uint32_t*)(y + d) = o_lo;
+      *(uint32_t*)(y + d + half) = o_hi;
+    };
+    const int items = rot_items + ((dim - rotary_dim) >> 1);  // per head: rotating items, then copying ones
+    for (int i = threadIdx.x; i < heads * items; i += 256) {
+      const int h = i / items, it = i - h * items;
+      head_item(qs + (int64_t)h * dim, qd + (int64_t)h * dim, it);
+    }
+    for (int i = threadIdx.x; i < heads_kv * items; i += 256) {
+      const int h = i / items, it = i - h * items;
+      head_item(ks + (int64_t)h * dim, kd + (int64_t)h * dim, it);
+    }
+    for (int64_t i = threadIdx.x * 2; i < kv_elems; i += 512) *(uint32_t*)(vd + i) = *(const uint32_t*)(vs + i);
+    return;
+  }
+  for (int64_t i = threadIdx.x; i < q_elems; i += 256) {
+    const int d = (int)(i % dim);
+    qd[i] = rotate(qs + (i - d), d);
+  }
+  for (int64_t i = threadIdx.x; i < kv_elems; i += 256) {
+    const int d = (int)(i % dim);
+    kd[i] = rotate(ks + (i - d), d);
+    vd[i] = vs[i];
+  }
+}
+
+const char* launch_rope_append_chunk(const void* q, const void* k_new, const void* v_new, void* q_rot, void* k_pages, void* v_pages,
+                                     const void* cos_table, const void* sin_table, const int32_t* cu_q,
+                                     const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, int batch,
+                                     int64_t total_q, int heads, int heads_kv, int dim, int rotary_dim, int64_t max_position,
+                                     int page_size, int64_t n_pages, int x_dtype, hipStream_t s) {
+  if (batch == 0 || total_q == 0) return nullptr;
+#define MI355_LAUNCH_ROPE(XT)                                                                                                   \
+  hipLaunchKernelGGL((rope_append_chunk_kernel<XT>), dim3((unsigned)total_q), dim3(256), 0, s, (const uint16_t*)q,              \
+                     (const uint16_t*)k_new, (const uint16_t*)v_new, (uint16_t*)q_rot, (uint16_t*)k_pages, (uint16_t*)v_pages,   \
+                     (const uint16_t*)cos_table, (const uint16_t*)sin_table, cu_q, cache_seqlens, block_table, bt_row_stride,   \
+                     batch, heads, heads_kv, dim, rotary_dim, max_position, page_size, n_pages)
+  if (x_dtype == MI355_DT_BF16) MI355_LAUNCH_ROPE(bf16_tag);
+  else MI355_LAUNCH_ROPE(fp16_tag);
+#undef MI355_LAUNCH_ROPE
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
 // Merge two attention results over disjoint key sets, given as fp32 rows with log2-domain log-sum-exp:
 //   out = (2^(lse_a - m) * o_a + 2^(lse_b - m) * o_b) / (2^(lse_a - m) + 2^(lse_b - m)),  m = max(lse_a, lse_b);
 // a row both sides left empty (-inf, -inf) becomes zero.  One thread per two head elements.

@@ -25,15 +25,17 @@ from . import native
 
 __all__ = [
     "AttentionCall", "DECODE_KEYS", "GQADecodeKernel", "GQADecodeMfmaKernel", "GQADecodePagedKernel",
-    "GQADecodePagedMfmaKernel", "GQAPrefillPagedWithFP8KVCacheFwdKernel", "GQAPrefillPagedWithKVCacheFwdKernel", "Kernel",
+    "GQADecodePagedMfmaKernel", "GQAPrefillPagedWithFP8KVCacheFwdKernel", "GQAPrefillPagedWithKVCacheFwdKernel",
+    "GQAPrefillPagedWithKVCacheRopeFwdKernel", "Kernel",
     "PAGED_DECODE_KEYS", "PAGED_PREFILL_KEYS", "PrefillCall",
     "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch",
 ]
 
 #: Dispatch keys of the paged decode ops, in no particular order (selection never reads the order).
 PAGED_DECODE_KEYS = ("gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel")
-#: Dispatch keys of the paged prefill op (the reference's third key, the fused-RoPE kernel, has no counterpart here).
-PAGED_PREFILL_KEYS = ("gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel", "gqa_prefill_paged_with_kv_cache_fwd_kernel")
+#: Dispatch keys of the paged prefill op (reference: src/tileops/ops/attention/selection.py:37-42).
+PAGED_PREFILL_KEYS = ("gqa_prefill_paged_with_kv_cache_rope_fwd_kernel", "gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel",
+                      "gqa_prefill_paged_with_kv_cache_fwd_kernel")
 #: Dispatch keys of the contiguous-cache decode op.
 DECODE_KEYS = ("gqa_decode_kernel", "gqa_decode_mfma_kernel")
 
@@ -494,7 +496,8 @@ class GQAPrefillPagedWithKVCacheFwdKernel(Kernel):
                 cos_table: Optional[torch.Tensor] = None, sin_table: Optional[torch.Tensor] = None) -> torch.Tensor:
         native.require_gfx950(q.device)
         if cos_table is not None or sin_table is not None:
-            raise NotImplementedError("fused RoPE is not served by the MI355X paged prefill kernels")
+            raise ValueError(f"{type(self).__name__} takes no rotary tables; the fused-RoPE call is served by "
+                             "GQAPrefillPagedWithKVCacheRopeFwdKernel")
         kernel = int(self.config.get("kernel", native.KERNEL_AUTO))
         nbytes = native.prefill_paged_workspace(self.batch, max_seqlen_q, q.shape[0], self.heads, self.heads_kv, self.dim,
                                                 self.page_size, block_table.shape[1], q.dtype, k_pages.dtype, kernel)
@@ -520,3 +523,49 @@ class GQAPrefillPagedWithFP8KVCacheFwdKernel(GQAPrefillPagedWithKVCacheFwdKernel
     @classmethod
     def applies(cls, call: PrefillCall) -> bool:
         return not call.fuse_rope and call.cache_dtype == torch.float8_e4m3fn
+
+
+
+class GQAPrefillPagedWithKVCacheRopeFwdKernel(GQAPrefillPagedWithKVCacheFwdKernel):
+    """The 16-bit-cache call with rotary position embedding fused in (reference:
+    src/tileops/kernels/attention/gqa_fwd.py:2020-2090 and the two TileLang kernels it launches, :1464-1582, :1660-1917):
+    query and new key rows are rotated (GPT-NeoX halves, position = cached length + index in the chunk), the rotated keys
+    are appended to the pages, attention runs over old + new tokens.  ``forward`` takes the cos/sin tables
+    ``[max_position, rotary_dim / 2]`` in the element type as its last two arguments."""
+
+    general = False
+
+    @classmethod
+    def applies(cls, call: PrefillCall) -> bool:
+        return bool(call.fuse_rope) and call.cache_dtype == call.dtype
+
+    def __init__(self, *, max_position: Optional[int] = None, rotary_dim: Optional[int] = None, **kwargs: Any) -> None:
+        super().__init__(max_position=max_position, rotary_dim=rotary_dim, **kwargs)
+        if rotary_dim is None or max_position is None:
+            raise ValueError("GQAPrefillPagedWithKVCacheRopeFwdKernel requires max_position and rotary_dim")
+        if rotary_dim <= 0 or rotary_dim % 2 != 0 or rotary_dim > self.dim:
+            raise ValueError("rotary_dim must be positive, even, and <= dim")
+        self.max_position, self.rotary_dim = max_position, rotary_dim
+
+    def forward(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pages: torch.Tensor,
+                v_pages: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
+                cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor, block_table: torch.Tensor, max_seqlen_q: int,
+                cos_table: Optional[torch.Tensor] = None, sin_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+        native.require_gfx950(q.device)
+        if cos_table is None or sin_table is None:
+            raise ValueError("the fused-RoPE prefill kernel needs cos_table and sin_table")
+        want = (self.max_position, self.rotary_dim // 2)
+        for name, t in (("cos_table", cos_table), ("sin_table", sin_table)):
+            if tuple(t.shape) != want or t.dtype != q.dtype or not t.is_contiguous() or t.device != q.device:
+                raise ValueError(f"{name} must be a contiguous {q.dtype} tensor of shape {want} on {q.device}, got "
+                                 f"{t.dtype} {tuple(t.shape)} on {t.device}")
+        kernel = int(self.config.get("kernel", native.KERNEL_AUTO))
+        nbytes = native.prefill_paged_rope_workspace(self.batch, max_seqlen_q, q.shape[0], self.heads, self.heads_kv, self.dim,
+                                                     self.page_size, block_table.shape[1], q.dtype, kernel)
+        out = torch.empty_like(q)
+        workspace = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+        native.prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q, cache_seqlens,
+                                  block_table, out, workspace, batch=self.batch, max_seqlen_q=max_seqlen_q, heads=self.heads,
+                                  heads_kv=self.heads_kv, dim=self.dim, page_size=self.page_size, rotary_dim=self.rotary_dim,
+                                  sm_scale=self.sm_scale, softcap=self.softcap, causal=self.is_causal, kernel=kernel)
+        return out

@@ -31,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "mi355_gqa_decode",
     "mi355_gqa_prefill_paged_workspace",
     "mi355_gqa_prefill_paged",
+    "mi355_gqa_prefill_paged_rope_workspace",
+    "mi355_gqa_prefill_paged_rope",
     "mi355_gather_probe",
     "mi355_kv_append_fp8",
 )
@@ -81,6 +83,16 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.mi355_gqa_prefill_paged.argtypes = [
         _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
         _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
+        _c_f32, _c_f32, _c_int, _c_int, _c_vp,
+    ]
+    lib.mi355_gqa_prefill_paged_rope_workspace.restype = _c_int
+    lib.mi355_gqa_prefill_paged_rope_workspace.argtypes = [
+        _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, ctypes.POINTER(_c_sz),
+    ]
+    lib.mi355_gqa_prefill_paged_rope.restype = _c_int
+    lib.mi355_gqa_prefill_paged_rope.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
+        _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_i64,
         _c_f32, _c_f32, _c_int, _c_int, _c_vp,
     ]
     lib.mi355_gather_probe.restype = _c_int
@@ -249,6 +261,33 @@ def prefill_paged(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_p
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
         batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, k_pages.shape[0], dtype_code(q.dtype),
         dtype_code(k_pages.dtype), float(sm_scale), float(softcap), int(bool(causal)), int(kernel), _stream_ptr(q.device)))
+
+
+def prefill_paged_rope_workspace(batch: int, max_seqlen_q: int, total_q: int, heads: int, heads_kv: int, dim: int, page_size: int,
+                                 max_pages_per_req: int, q_dtype: torch.dtype, kernel: int = KERNEL_AUTO) -> int:
+    """Workspace bytes of a paged prefill call with fused rotary embedding.  Touches no device."""
+    lib = load()
+    nbytes = _c_sz(0)
+    _check(lib.mi355_gqa_prefill_paged_rope_workspace(
+        batch, max_seqlen_q, total_q, heads, heads_kv, dim, page_size, max_pages_per_req, dtype_code(q_dtype), kernel,
+        ctypes.byref(nbytes)))
+    return int(nbytes.value)
+
+
+def prefill_paged_rope(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                       cos_table: torch.Tensor, sin_table: torch.Tensor, cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor,
+                       block_table: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, *, batch: int, max_seqlen_q: int,
+                       heads: int, heads_kv: int, dim: int, page_size: int, rotary_dim: int, sm_scale: float, softcap: float,
+                       causal: bool, kernel: int = KERNEL_AUTO) -> None:
+    """Enqueue one paged prefill call with fused rotary embedding (rotate q and k_new, append, attention)."""
+    lib = load()
+    _check(lib.mi355_gqa_prefill_paged_rope(
+        q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), cos_table.data_ptr(),
+        sin_table.data_ptr(), cu_seqlens_q.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        out.data_ptr(), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, k_pages.shape[0], dtype_code(q.dtype),
+        int(rotary_dim), int(cos_table.shape[0]), float(sm_scale), float(softcap), int(bool(causal)), int(kernel),
+        _stream_ptr(q.device)))
 
 
 def gather_probe(cache: torch.Tensor, seqlens: torch.Tensor, block_table: torch.Tensor, page_size: int, max_len: int) -> torch.Tensor:

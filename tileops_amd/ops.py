@@ -27,6 +27,7 @@ from .backend import Target
 from .kernels import (
     DECODE_KEYS, PAGED_DECODE_KEYS, PAGED_PREFILL_KEYS, AttentionCall, GQADecodeKernel, GQADecodeMfmaKernel,
     GQADecodePagedKernel, GQADecodePagedMfmaKernel, GQAPrefillPagedWithFP8KVCacheFwdKernel,
+    GQAPrefillPagedWithKVCacheRopeFwdKernel,
     GQAPrefillPagedWithKVCacheFwdKernel, PrefillCall, get_arch,
 )
 from .op_base import _UNRESOLVED, Op
@@ -382,8 +383,9 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
     Keeps the reference op's contract (src/tileops/ops/attention/gqa.py:765-1157): constructor arguments, defaults and
     messages, the eleven ``forward`` arguments in order, the validation of devices, contiguity, shapes, dtypes, scale
     values, ``cu_seqlens_q`` / ``cache_seqlens`` consistency, capacity and block-table range (:897-1046; like the
-    reference it reads a few device scalars to do so).  ``fuse_rope=True`` is accepted by the constructor's checks as in
-    the reference but no kernel here serves it: such an op raises when called.
+    reference it reads a few device scalars to do so).  With ``fuse_rope=True`` (16-bit cache only, as in the reference)
+    query and new key rows are rotated at their logical positions before the append; the cos/sin tables are built once
+    per (device, dtype) like the reference's (:1048-1065, src/tileops/ops/rope.py:97-120).
     """
 
     def __init__(self, batch: int, heads: int, heads_kv: int, max_pages_per_req: int, page_size: int, dim: int,
@@ -414,6 +416,7 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
         self.sm_scale = _attention_scale(dim, sm_scale)
         self.softcap = _score_softcap(softcap)
         self.fuse_rope, self.rope_base, self.max_position, self.rotary_dim = fuse_rope, rope_base, max_position, rotary_dim
+        self._rope_cos_cache: Dict[tuple, tuple] = {}
         self.tune = tune
         if target is not None:
             self.target = target
@@ -422,9 +425,24 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
     @property
     def default_kernel_map(self) -> Dict[str, type]:
         return {
+            "gqa_prefill_paged_with_kv_cache_rope_fwd_kernel": GQAPrefillPagedWithKVCacheRopeFwdKernel,
             "gqa_prefill_paged_with_kv_cache_fwd_kernel": GQAPrefillPagedWithKVCacheFwdKernel,
             "gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel": GQAPrefillPagedWithFP8KVCacheFwdKernel,
         }
+
+    def _rope_tables(self, device: torch.device, dtype: torch.dtype) -> "tuple[Optional[torch.Tensor], Optional[torch.Tensor]]":
+        """cos/sin ``[max_position, rotary_dim / 2]`` in *dtype*: angle = position * base**(-i / half), computed in fp32
+        (src/tileops/ops/rope.py:116-120), cached per (device, dtype) (gqa.py:1048-1065)."""
+        if not self.fuse_rope:
+            return None, None
+        cached = self._rope_cos_cache.get((device, dtype))
+        if cached is None:
+            half = self.rotary_dim // 2
+            freqs = 1.0 / (self.rope_base ** (torch.arange(0, half, device=device, dtype=torch.float32) / half))
+            angles = torch.outer(torch.arange(self.max_position, device=device, dtype=torch.float32), freqs)
+            cached = (torch.cos(angles).to(dtype).contiguous(), torch.sin(angles).to(dtype).contiguous())
+            self._rope_cos_cache[(device, dtype)] = cached
+        return cached
 
     def _resolved_cache_dtype(self, dtype: torch.dtype) -> torch.dtype:
         return dtype if self.cache_dtype is None else self.cache_dtype
@@ -519,6 +537,9 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
         if max_total_len > self.max_cache_len:
             raise ValueError("cache_seqlens + q_len exceeds paged KV capacity: "
                              f"max total length {max_total_len}, capacity {self.max_cache_len}")
+        if self.fuse_rope and max_total_len > self.max_position:
+            raise ValueError("cache_seqlens + q_len exceeds RoPE max_position: "
+                             f"max total length {max_total_len}, max_position {self.max_position}")
         num_pages = k_pages.shape[0] // self.page_size
         min_page, max_page = int(block_table.min().item()), int(block_table.max().item())
         if min_page < 0:
@@ -540,7 +561,8 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
         inputs = (q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table)
         call = self.attention_call(q.dtype, q.device)
         key = self.select_kernel_key(PAGED_PREFILL_KEYS, call)
-        return self._get_kernel(inputs, key, call)(*inputs, max_seqlen_q)
+        cos_table, sin_table = self._rope_tables(q.device, q.dtype)
+        return self._get_kernel(inputs, key, call)(*inputs, max_seqlen_q, cos_table, sin_table)
 
     @property
     def total_flops(self) -> int:

@@ -226,7 +226,7 @@ class _PrefillView:
         self.row, self.dtype = dict(row), dtype
 
     def eval_roofline(self) -> tuple[int, int]:
-        return gqa_prefill_paged_with_kv_cache_fwd_roofline(dtype=self.dtype, **{k: v for k, v in self.row.items() if k not in ("dtypes", "label")})
+        return gqa_prefill_paged_with_kv_cache_fwd_roofline(dtype=self.dtype, **{k: v for k, v in self.row.items() if k not in ("dtypes", "label", "fuse_rope", "max_position", "rotary_dim", "rope_base")})
 
 
 def _prefill_case(row: dict, dtype: torch.dtype, device: torch.device):
@@ -238,7 +238,8 @@ def _prefill_case(row: dict, dtype: torch.dtype, device: torch.device):
     total_q = sum(q_lens)
     op = GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(
         batch=batch, heads=heads, heads_kv=heads_kv, max_pages_per_req=max_pages, page_size=page, dim=dim,
-        is_causal=row.get("is_causal", True), cache_dtype=cache_dtype if cache_dtype == FP8 else None, softcap=row.get("softcap"))
+        is_causal=row.get("is_causal", True), cache_dtype=cache_dtype if cache_dtype == FP8 else None, softcap=row.get("softcap"),
+        fuse_rope=bool(row.get("fuse_rope", False)), max_position=row.get("max_position"), rotary_dim=row.get("rotary_dim"))
     fp8 = cache_dtype == FP8
     amp = 0.5 if fp8 else 1.0
     q = torch.randn(total_q, heads, dim, device=device, dtype=dtype)
