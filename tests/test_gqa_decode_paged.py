@@ -115,7 +115,7 @@ def test_gqa_decode_paged_bs1_both_tiers(real_len, reverse_pages):
 )
 def test_gqa_decode_paged_dispatch_lands_on_a_kernel_that_serves_the_call(batch, dtype, dim, page_size, softcap):
     """Every shape of the reference's dispatch table is served: by the specialised kernel inside its region,
-    by the general one elsewhere (head_dim 64 is outside the MFMA region)."""
+    by the general one elsewhere (head dims 64 and 128 are inside the MFMA region, page 192 is not)."""
     require_gfx950()
     seqlen_kv = 8064 if page_size == 192 else 8192
     op = PagedOp(batch, 32, 4, seqlen_kv, dim, page_size, softcap=softcap)
@@ -123,8 +123,7 @@ def test_gqa_decode_paged_dispatch_lands_on_a_kernel_that_serves_the_call(batch,
     call = op.attention_call(dtype, None, torch.device(DEV, 0))
     expected = "GQADecodePagedMfmaKernel" if op.kernel_map["gqa_decode_paged_mfma_kernel"].applies(call) else "GQADecodePagedKernel"
     assert kernel.__class__.__name__ == expected
-    if dim == 64:
-        assert expected == "GQADecodePagedKernel"
+    assert expected == "GQADecodePagedMfmaKernel"  # head dims 64 and 128, pages of 16 or a multiple of 32 tokens
 
 
 # --- beyond the reference's coverage ------------------------------------------------------------------------
@@ -260,21 +259,24 @@ def test_multi_token_causal_chunk(kernel_key, fp8, q_len, is_causal):
         pytest.param(40, 16, 2, id="rows320-ten-row-groups"),
     ],
 )
-def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, heads, heads_kv):
+@pytest.mark.parametrize("dim", [128, 64])
+def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, heads, heads_kv, dim):
     """More than 32 query rows per kv head: the row groups of a kv head run as 2, 4 or 8 waves around one LDS ring (or
     fall back to one wave of four row blocks when their number is odd).  Ragged lengths so that partitions start and
     end inside sequences, tails shorter than a tile, a sequence shorter than the chunk, NaN in every unaddressed token;
     head counts that leave the grid with workgroups past the last (partition, kv head)."""
     require_gfx950()
+    if fp8 and dim != 128:
+        pytest.skip("the fp8 MFMA path is head dim 128 only")
     lens = [2100, q_len, q_len + 33, 700, q_len + 31, q_len + 1]
-    case = _ragged_case(len(lens), heads, heads_kv, 128, 64, lens, dtype, q_len=q_len, fp8=fp8, seed=31)
-    op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], 128, 64, is_causal=True)
+    case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, dtype, q_len=q_len, fp8=fp8, seed=31)
+    op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], dim, 64, is_causal=True)
     if not _serves(op, "gqa_decode_paged_mfma_kernel", dtype, fp8):
         pytest.skip("the MFMA kernel does not serve this shape")
     _force(op, "gqa_decode_paged_mfma_kernel")
     out = _run_and_compare(op, case, 64, tol, is_causal=True)
     # and against the other implementation, which shares none of the tiling
-    other = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], 128, 64, is_causal=True)
+    other = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], dim, 64, is_causal=True)
     if _serves(other, "gqa_decode_paged_kernel", dtype, fp8):
         _force(other, "gqa_decode_paged_kernel")
         dev = [None if t is None else t.to(DEV) for t in case]

@@ -81,7 +81,7 @@ int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_s
   } else {
     plan->max_splits = 0;
     plan->split_tokens = 0;
-    plan->n_parts = mfma_num_parts(heads_kv, rows, kv_dtype);
+    plan->n_parts = mfma_num_parts(heads_kv, rows, dim, kv_dtype);
     size_t total = mfma_workspace_bytes(plan->n_parts, heads_kv, rows, dim, batch);
     plan->part_o_bytes = total;  // the MFMA launcher lays out its own workspace
     plan->part_lse_bytes = 0;

@@ -87,7 +87,7 @@ __host__ __device__ inline void split_geometry(int len, int split_tokens, int ma
 const char* launch_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
 const char* launch_generic_combine(const DecodeParams& p, int q_dtype, hipStream_t s);
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap);
-int mfma_num_parts(int heads_kv, int rows, int kv_dtype);
+int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype);
 size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int batch);
 const char* launch_mfma(const DecodeParams& p, int q_dtype, int kv_dtype, bool skip_combine, hipStream_t s);
 const char* launch_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,

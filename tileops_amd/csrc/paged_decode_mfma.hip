@@ -43,7 +43,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 #define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
-constexpr int kD = 128;       // head dim served by this kernel
+constexpr int kD = 128;       // head dim of the fp8 path (16-bit caches also run 64)
 constexpr int kNumCU = 256;   // MI355X
 constexpr bool kLateIssueFp8 = true;
 
@@ -53,9 +53,10 @@ __host__ __device__ constexpr int row_groups(int rows, int nrb) { return (rows +
 __host__ __device__ constexpr int ring_row_groups(int rows, int nrb, int shw) { return (row_groups(rows, nrb) + shw - 1) / shw * shw; }
 constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
-template <typename KVT> struct Geom {
+template <typename KVT, int D = kD> struct Geom {
   static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
-  static constexpr int ROW = kD * ElemTraits<KVT>::bytes;  // bytes of one (token, kv head) row
+  static_assert(D == 128 || (!FP8 && D == 64), "head dim 128, or 64 with a 16-bit cache");
+  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 256, or 128 (fp8; 16-bit head dim 64)
   static constexpr int TPI = 1024 / ROW;                   // tokens per direct-to-LDS instruction
   static constexpr int NI = kCT / TPI;                     // instructions per K (or V) stage
   static constexpr int KBYTES = kCT * ROW;
@@ -217,15 +218,19 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // serve SHW consecutive row groups of the same (partition, kv head), i.e. they walk the same tiles.  They share one
 // LDS ring: each fetches 1/SHW of every stage, and one barrier per tile makes all parts visible and retires the slot
 // that is refilled next.  All waves execute the same number of barriers because they own the same tile range.
-template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW>
+template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW, int D>
 __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
-  using G = Geom<KVT>;
+  using G = Geom<KVT, D>;
   constexpr bool FP8 = G::FP8;
+  constexpr int NJ = D / 32;    // 32-wide steps of the head dim in Q.K^T
+  constexpr int NDB = D / 16;   // 16-wide blocks of the head dim in the output
+  constexpr bool ROW128 = G::ROW == 128;        // 128-byte rows: fp8, or 16-bit with head dim 64 (8 KiB stages, eight waves a CU)
+  constexpr bool R128 = ROW128 && !FP8;         // 16-bit rows of 128 bytes: the fp8 K layout with 16-bit elements
   constexpr bool SH = SHW > 1;
   static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
   // or after it (a tile lands before the next is requested: fewer requests in flight per compute unit).
-  constexpr bool LATE = SH || (FP8 && NRB == 1 && kLateIssueFp8);
+  constexpr bool LATE = SH || (Geom<KVT, D>::ROW == 128 && NRB == 1 && kLateIssueFp8);
   constexpr int NIW = G::NI / SHW;                     // K (or V) fetch instructions per stage issued by this wave
   constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -353,32 +358,43 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
   // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
   // t = i*TPI + l/LPT (LPT lanes per token row), 16-byte slot l%LPT of that row.  The chunk fetched into
   // slot s of token t is s ^ f(t), with f chosen per operand so that the MFMA-layout reads are conflict free:
-  //   bf16 K: f = t%16          bf16 V: f = 2*(t%8)
-  //   fp8  K: f = (t/2)%8       fp8  V: f = (t/2)%4 + 4*((t/16)%2)
+  //   16-bit, 256-byte rows  K: f = t%16       V: f = 2*(t%8)
+  //   16-bit, 128-byte rows  K: f = (t/2)%8    V: f = 2*((t/2)%4)
+  //   fp8 (128-byte rows)    K: f = (t/2)%8    V: f = (t/2)%4 + 4*((t/16)%2)
   constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
-  // The patterns repeat every 4 (bf16 K), 2 (bf16 V, fp8 K) instructions, or change once half way (fp8 V): a wave
-  // keeps one offset register per distinct pattern among the instructions it issues.
+  // With 256-byte rows the patterns repeat every 4 (K) and 2 (V) instructions; with 128-byte rows every 2 (K), and V
+  // is the same for all (16-bit) or changes once half way (fp8).  A wave keeps one offset register per distinct
+  // pattern among the instructions it issues.
   const int ts = lane / LPT, slot = lane % LPT;
-  constexpr int NKO = NIW < (FP8 ? 2 : 4) ? NIW : (FP8 ? 2 : 4);
-  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (NIW < 2 ? NIW : 2);
+  constexpr int NKO = NIW < (ROW128 ? 2 : 4) ? NIW : (ROW128 ? 2 : 4);
+  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < 2 ? NIW : 2));
   uint32_t voff_k[NKO], voff_v[NVO];
 #pragma unroll
   for (int e = 0; e < NKO; e++) {
     const int i = i0 + e;
-    voff_k[e] = ts * row_stride + (FP8 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((4 * i + ts) & 15)) << 4));
+    voff_k[e] = ts * row_stride + (ROW128 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((4 * i + ts) & 15)) << 4));
   }
 #pragma unroll
   for (int e = 0; e < NVO; e++) {
     const int i = FP8 ? (NIW == 4 ? 2 * e : i0) : i0 + e;
-    voff_v[e] = ts * row_stride + (FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4) : ((slot ^ (2 * ((4 * i + ts) & 7))) << 4));
+    voff_v[e] = ts * row_stride + (FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4)
+                                      : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((4 * i + ts) & 7))) << 4)));
   }
   auto k_sel = [](int ii) __attribute__((always_inline)) { return ii % NKO; };
   auto v_sel = [](int ii) __attribute__((always_inline)) { return FP8 ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
-  constexpr int NKA = FP8 ? 2 : 4;
-  uint32_t kaddr[NKA], vaddr[8];
-  if (!FP8) {
+  constexpr int NKA = ROW128 ? 2 : 4;
+  uint32_t kaddr[NKA], vaddr[NDB];
+  if constexpr (R128) {
+    // head dim 64: K rows of 128 bytes read exactly like the fp8 K rows (16-byte chunk g + 4j of row c), V^T like the
+    // 256-byte-row case with four 32-byte slots per row instead of eight
+#pragma unroll
+    for (int j = 0; j < 2; j++) kaddr[j] = lds_wave + (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
+    const int tk = 4 * g + c / 4;
+#pragma unroll
+    for (int db = 0; db < NDB; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 128 + ((tk >> 1) & 3) * 32 + (c & 3) * 8) ^ (db * 32));
+  } else if constexpr (!FP8) {
 #pragma unroll
     for (int j = 0; j < 4; j++) kaddr[j] = lds_wave + (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
     const int tk = 4 * g + c / 4;  // transpose read: lane supplies row tk, 8 bytes at column group c%4
@@ -489,8 +505,8 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
   };
 
   // ---- per-segment state ----------------------------------------------------------------------------------
-  u32x4 qreg[NRB][4];
-  f32x4 o_acc[NRB][8];
+  u32x4 qreg[NRB][NJ];
+  f32x4 o_acc[NRB][NDB];
   float m_run[NRB], l_run[NRB];
   int limit[NRB];
   const int qoff = (p.causal && p.q_len > 1) ? p.q_len - 1 : 0;
@@ -507,9 +523,9 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
       int r = rg * (16 * NRB) + rb * 16 + c;
       bool valid = r < seg_q_len * p.group;
       int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
-      const char* qp = (const char*)p.q + (((seg_q_row0 + s) * p.heads + kvh * p.group + gi) * kD) * 2;
+      const char* qp = (const char*)p.q + (((seg_q_row0 + s) * p.heads + kvh * p.group + gi) * D) * 2;
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
+      for (int j = 0; j < NJ; j++) {
         // head elements this lane contributes to k-step j: 8 consecutive ones, matching the K operand
         int d0 = FP8 ? 64 * (j >> 1) + 16 * g + 8 * (j & 1) : 32 * j + 8 * g;
         u32x4 z = {0, 0, 0, 0};
@@ -519,7 +535,7 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
       m_run[rb] = kNegFloor;
       l_run[rb] = 0.f;
 #pragma unroll
-      for (int db = 0; db < 8; db++) o_acc[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int db = 0; db < NDB; db++) o_acc[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     // Make the query loads land here: an empty asm that "modifies" each register forces the compiler to put
     // its own vmcnt wait in this (rare) block instead of in the steady-state loop, where such a wait would
@@ -527,7 +543,7 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
+      for (int j = 0; j < NJ; j++) {
         asm volatile("" : "+v"(qreg[rb][j]));
         // a negative softmax scale is carried by the query (an exact sign flip), so the scale itself is positive
         qreg[rb][j] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
@@ -544,24 +560,25 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
   // With an fp8 cache and several row blocks registers are short: V^T then stays in bytes until the PV product
   // consumes it (widened one 16-column block at a time, in between the MFMAs).
   constexpr bool LATE_V = FP8 && NRB >= 2;
-  u32x4 va_op[LATE_V ? 1 : 8];
+  u32x4 va_op[LATE_V ? 1 : NDB];
   i32x2 vraw[LATE_V ? 8 : 1];
   u32x4 pk[NRB];
   float alpha[NRB];
   auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
-    u32x4 ka_op[2][4];
+    u32x4 ka_op[2][NJ];
     f32x4 ksc[2], vsc[2];
-    if (!FP8) {
+    constexpr uint32_t HALF = 16 * G::ROW;  // bytes of one 16-token block of K (or V)
+    if constexpr (!FP8) {
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j] + (SOFF + tb * 4096));
+        for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j] + (SOFF + tb * HALF));
 #pragma unroll
-      for (int db = 0; db < 8; db++) {
+      for (int db = 0; db < NDB; db++) {
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + SOFF));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + (SOFF + 4096)));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + (SOFF + HALF)));
         u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
         va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
       }
@@ -601,7 +618,7 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NJ; j++)
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
@@ -671,14 +688,14 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-      for (int db = 0; db < 8; db++) {
+      for (int db = 0; db < NDB; db++) {
         o_acc[rb][db] *= alpha[rb];  // alpha is 1 for rows that kept their reference
         __builtin_amdgcn_sched_barrier(0);  // one tile at a time: keeps the copies out of the accumulation registers short-lived
       }
   };
   auto value_step = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int db = 0; db < 8; db++) {
+    for (int db = 0; db < NDB; db++) {
       u32x4 vt;
       if constexpr (LATE_V) vt = widen8<QT>((uint32_t)vraw[db][0], (uint32_t)vraw[db][1]);
       else vt = va_op[db];
@@ -699,13 +716,13 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
         const int64_t orow = (seg_q_row0 + s) * p.heads + kvh * p.group + gi;
         if (p.final_o) {  // fp32 rows + LSE for a later merge with another call
 #pragma unroll
-          for (int db = 0; db < 8; db++) *(f32x4*)(p.final_o + orow * kD + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+          for (int db = 0; db < NDB; db++) *(f32x4*)(p.final_o + orow * D + 16 * db + 4 * g) = o_acc[rb][db] * inv;
           if (g == 0) p.final_lse[orow] = l_tot > 0.f ? m_run[rb] + log2f(l_tot) : -INFINITY;
           continue;
         }
-        uint16_t* op = (uint16_t*)p.out + orow * kD;
+        uint16_t* op = (uint16_t*)p.out + orow * D;
 #pragma unroll
-        for (int db = 0; db < 8; db++) {
+        for (int db = 0; db < NDB; db++) {
           f32x4 o = o_acc[rb][db] * inv;
           u32x2 w;
           w[0] = Mma<QT>::pack(o[0], o[1]);
@@ -714,9 +731,9 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
         }
       } else {
         int64_t grow = ((int64_t)(2 * part + which) * p.heads_kv + kvh) * p.rows + r;
-        float* pp = p.part_o + grow * kD;
+        float* pp = p.part_o + grow * D;
 #pragma unroll
-        for (int db = 0; db < 8; db++) *(f32x4*)(pp + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+        for (int db = 0; db < NDB; db++) *(f32x4*)(pp + 16 * db + 4 * g) = o_acc[rb][db] * inv;
         if (g == 0) p.part_lse[grow] = l_tot > 0.f ? m_run[rb] + log2f(l_tot) : -INFINITY;
       }
     }
@@ -855,10 +872,15 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
   const int s = r / p.group, gi = r - s * p.group;
   if (p.cu_q && r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
   const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
-  uint32_t* op = (uint32_t*)((uint16_t*)p.out + orow * kD) + lane;
+  // every lane owns two head elements; with head dim 64 the upper half of the wave idles (reads element 0, stores nothing)
+  const int hd = p.dim;
+  const bool owns = 2 * lane < hd;
+  const int dl = owns ? 2 * lane : 0;
+  uint32_t* op = (uint32_t*)((uint16_t*)p.out + orow * hd) + (dl >> 1);
   auto store = [&](float a0, float a1, float lse) {
+    if (!owns) return;
     if (p.final_o) {
-      *(f32x2*)(p.final_o + orow * kD + 2 * lane) = f32x2{a0, a1};
+      *(f32x2*)(p.final_o + orow * hd + dl) = f32x2{a0, a1};
       if (lane == 0) p.final_lse[orow] = lse;
     } else {
       *op = Mma<QT>::pack(a0, a1);
@@ -885,7 +907,7 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
   // this wave's first eight partial rows go out together with the LSEs, before any weight is known
   f32x2 rows[PRE];
 #pragma unroll
-  for (int i = 0; i < PRE; i++) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + wave + nw * i, p_last)) * kD + 2 * lane);
+  for (int i = 0; i < PRE; i++) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + wave + nw * i, p_last)) * hd + dl);
   // lane i keeps the LSE of partition i of the first 64 (all of them, as a rule); further ones are re-read
   const float lse0 = (p_first + lane <= p_last && owns_tiles(p_first + lane)) ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
   float M = lse0;
@@ -920,7 +942,7 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
         const int idx = wave + nw * (i0 + i), pp = p_first + idx;  // wave-uniform
         if (idx < 64) wt[i] = __shfl(w0, idx, 64);
         else wt[i] = (pp <= p_last && owns_tiles(pp)) ? fast_exp2(p.part_lse[slot_of(pp)] - M) : 0.f;
-        if (i0 > 0) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(pp, p_last)) * kD + 2 * lane);
+        if (i0 > 0) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(pp, p_last)) * hd + dl);
       }
 #pragma unroll
       for (int i = 0; i < PRE; i++)
@@ -948,7 +970,7 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
 
-template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW>
+template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW, int D>
 const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   const int n_rg = ring_row_groups(p.rows, NRB, SHW);
   const int64_t waves = (int64_t)p.n_parts * p.heads_kv * n_rg;
@@ -956,8 +978,8 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   // shared-stage variant: 8 XCDs x (workgroups of a group) x ceil(groups / 8), a group being one (partition, kv head);
   // the workgroups of groups past the last exit at once
   const int grid = SH ? 8 * (n_rg / SHW) * ((p.n_parts * p.heads_kv + 7) / 8) : (int)((waves + NW - 1) / NW);
-  const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT>::STAGE;
-  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SHW>;
+  const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT, D>::STAGE;
+  auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SHW, D>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
   static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
   int dev = 0;
@@ -988,26 +1010,27 @@ int row_blocks_for(int rows) { return rows <= 16 ? 1 : 2; }
 // fetch instructions per wave, one trip through the memory system per tile); an odd count is rounded up by one idle
 // row group.  Eight waves a compute unit either way (accumulators of two row blocks fit ordinary vector registers);
 // the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
-int ring_waves_for(int rows, bool fp8) {
+// (narrow = 128-byte rows, fp8 or head dim 64: four fetch instructions per K tile, so at most four waves share them)
+int ring_waves_for(int rows, bool narrow) {
   const int n = row_groups(rows, 2);
   if (rows <= 32) return 1;
   const int even = (n + 1) / 2 * 2;
-  if (even % 8 == 0 && !fp8) return 8;
+  if (even % 8 == 0 && !narrow) return 8;
   if (even % 4 == 0) return 4;
   return 2;
 }
 
-template <typename QT, typename KVT>
+template <typename QT, typename KVT, int D>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  constexpr bool FP8 = Geom<KVT>::FP8;
-  if (row_blocks_for(p.rows) == 1) return launch_t4<QT, KVT, 1, 2, FP8 ? 8 : 4, 1>(p, ws_prefix, skip_combine, s);
-  switch (ring_waves_for(p.rows, FP8)) {
-    case 1: return launch_t4<QT, KVT, 2, 2, FP8 ? 8 : 4, 1>(p, ws_prefix, skip_combine, s);
-    case 2: return launch_t4<QT, KVT, 2, FP8 ? 4 : 2, 2, 2>(p, ws_prefix, skip_combine, s);
-    case 4: return launch_t4<QT, KVT, 2, 4, 4, 4>(p, ws_prefix, skip_combine, s);
+  constexpr bool SMALL = Geom<KVT, D>::ROW == 128;  // 8 KiB stages: eight unshared waves a CU, four-deep pair rings
+  if (row_blocks_for(p.rows) == 1) return launch_t4<QT, KVT, 1, 2, SMALL ? 8 : 4, 1, D>(p, ws_prefix, skip_combine, s);
+  switch (ring_waves_for(p.rows, SMALL)) {
+    case 1: return launch_t4<QT, KVT, 2, 2, SMALL ? 8 : 4, 1, D>(p, ws_prefix, skip_combine, s);
+    case 2: return launch_t4<QT, KVT, 2, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
+    case 4: return launch_t4<QT, KVT, 2, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
     default:
-      if constexpr (!FP8) return launch_t4<QT, KVT, 2, 4, 8, 8>(p, ws_prefix, skip_combine, s);
-      return "MFMA kernel: no ring of eight waves for an fp8 cache";
+      if constexpr (!SMALL) return launch_t4<QT, KVT, 2, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      return "MFMA kernel: no ring of eight waves with 128-byte rows";
   }
 }
 
@@ -1017,21 +1040,22 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap) {
   (void)q_len; (void)heads; (void)heads_kv; (void)softcap;
-  if (dim != kD) return false;
+  const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
+  if (!(dim == 128 || (dim == 64 && !fp8))) return false;
   if (!(page_size == 16 || page_size % kCT == 0)) return false;
-  if (kv_dtype != MI355_DT_FP8_E4M3FN && kv_dtype != q_dtype) return false;
+  if (!fp8 && kv_dtype != q_dtype) return false;
   return true;
 }
 
 // Number of equal ranges the tile stream is cut into: one wave per (range, kv head, row group), sized so
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
-int mfma_num_parts(int heads_kv, int rows, int kv_dtype) {
+int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  const int nrb = row_blocks_for(rows), shw = ring_waves_for(rows, fp8);
+  const int nrb = row_blocks_for(rows), shw = ring_waves_for(rows, fp8 || dim == 64);
   const int n_rg = ring_row_groups(rows, nrb, shw);
-  // resident waves per CU: eight with an fp8 cache (LDS-limited) and for shared rings (accumulators in ordinary
+  // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
-  const int waves_per_cu = (fp8 || shw > 1) ? 8 : 4;
+  const int waves_per_cu = (fp8 || dim == 64 || shw > 1) ? 8 : 4;
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
@@ -1054,15 +1078,21 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
   char* ws = (char*)p_in.part_o;
   p.part_o = (float*)ws;
-  p.part_lse = (float*)(ws + align256(slots * kD * sizeof(float)));
-  int* ws_prefix = (int*)(ws + align256(slots * kD * sizeof(float)) + align256(slots * sizeof(float)));
+  p.part_lse = (float*)(ws + align256(slots * p.dim * sizeof(float)));
+  int* ws_prefix = (int*)(ws + align256(slots * p.dim * sizeof(float)) + align256(slots * sizeof(float)));
   // the kernel addresses pool rows with 32 bits
   const int64_t pool_rows = p.kv_starts ? INT32_MAX - 1 : (p.contig_stride ? (int64_t)p.batch * p.contig_stride : p.n_pages * p.page_size);
   if (pool_rows >= INT32_MAX) return "MFMA kernel: the KV pool has 2^31 or more rows";
-  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag>(p, ws_prefix, skip_combine, s);
-  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag>(p, ws_prefix, skip_combine, s);
-  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag>(p, ws_prefix, skip_combine, s);
-  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag>(p, ws_prefix, skip_combine, s);
+  if (p.dim == 64) {
+    if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 64>(p, ws_prefix, skip_combine, s);
+    if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 64>(p, ws_prefix, skip_combine, s);
+    return "MFMA kernel: head dim 64 needs a 16-bit cache of the query's element type";
+  }
+  if (p.dim != 128) return "MFMA kernel: unsupported head dim";
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 128>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 128>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag, 128>(p, ws_prefix, skip_combine, s);
+  if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag, 128>(p, ws_prefix, skip_combine, s);
   return "MFMA kernel: unsupported (q_dtype, kv_dtype) pair";
 }
 
