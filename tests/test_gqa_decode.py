@@ -93,14 +93,14 @@ def test_gqa_decode_kernel_rejects(args, match):
 
 @pytest.mark.gpu
 def test_gqa_decode_dispatch():
-    """Head dims 128 and 64 select the MFMA kernel for every dtype and batch; other head dims fall back to the general one."""
+    """Head dims 64, 128 and 256 select the MFMA kernel for every dtype and batch."""
     require_gfx950()
     q = torch.empty(1, device=DEV)
     op = DecodeOp(1, 32, 4, 8192, 128)
     assert op._get_kernel((q,), torch.float16).__class__.__name__ == "GQADecodeMfmaKernel"
     assert op._get_kernel((q,), torch.bfloat16).__class__.__name__ == "GQADecodeMfmaKernel"
     assert DecodeOp(4, 32, 4, 4096, 64)._get_kernel((q,), torch.float16).__class__.__name__ == "GQADecodeMfmaKernel"
-    assert DecodeOp(4, 32, 4, 4096, 256)._get_kernel((q,), torch.float16).__class__.__name__ == "GQADecodeKernel"
+    assert DecodeOp(4, 32, 4, 4096, 256)._get_kernel((q,), torch.float16).__class__.__name__ == "GQADecodeMfmaKernel"
 
 
 @pytest.mark.gpu

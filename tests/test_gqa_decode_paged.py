@@ -123,7 +123,7 @@ def test_gqa_decode_paged_dispatch_lands_on_a_kernel_that_serves_the_call(batch,
     call = op.attention_call(dtype, None, torch.device(DEV, 0))
     expected = "GQADecodePagedMfmaKernel" if op.kernel_map["gqa_decode_paged_mfma_kernel"].applies(call) else "GQADecodePagedKernel"
     assert kernel.__class__.__name__ == expected
-    assert expected == "GQADecodePagedMfmaKernel"  # head dims 64 and 128, pages of 16 or a multiple of 32 tokens
+    assert expected == "GQADecodePagedMfmaKernel"  # head dims 64, 128, 256; pages of 16 or a multiple of 32 tokens
 
 
 # --- beyond the reference's coverage ------------------------------------------------------------------------
@@ -259,7 +259,7 @@ def test_multi_token_causal_chunk(kernel_key, fp8, q_len, is_causal):
         pytest.param(40, 16, 2, id="rows320-ten-row-groups"),
     ],
 )
-@pytest.mark.parametrize("dim", [128, 64])
+@pytest.mark.parametrize("dim", [128, 64, 256])
 def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, heads, heads_kv, dim):
     """More than 32 query rows per kv head: the row groups of a kv head run as 2, 4 or 8 waves around one LDS ring (or
     fall back to one wave of four row blocks when their number is odd).  Ragged lengths so that partitions start and

@@ -43,7 +43,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 #define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
-constexpr int kD = 128;       // head dim of the fp8 path (16-bit caches also run 64)
+constexpr int kD = 128;       // head dim of the fp8 path (16-bit caches also run 64 and 256)
 constexpr int kNumCU = 256;   // MI355X
 constexpr bool kLateIssueFp8 = true;
 
@@ -55,8 +55,8 @@ constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT, int D = kD> struct Geom {
   static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
-  static_assert(D == 128 || (!FP8 && D == 64), "head dim 128, or 64 with a 16-bit cache");
-  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 256, or 128 (fp8; 16-bit head dim 64)
+  static_assert(D == 128 || (!FP8 && (D == 64 || D == 256)), "head dim 128, or 64 / 256 with a 16-bit cache");
+  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 128 (fp8; 16-bit head dim 64), 256 or 512
   static constexpr int TPI = 1024 / ROW;                   // tokens per direct-to-LDS instruction
   static constexpr int NI = kCT / TPI;                     // instructions per K (or V) stage
   static constexpr int KBYTES = kCT * ROW;
@@ -219,7 +219,7 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // LDS ring: each fetches 1/SHW of every stage, and one barrier per tile makes all parts visible and retires the slot
 // that is refilled next.  All waves execute the same number of barriers because they own the same tile range.
 template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW, int D>
-__global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+__global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT, D>;
   constexpr bool FP8 = G::FP8;
   constexpr int NJ = D / 32;    // 32-wide steps of the head dim in Q.K^T
@@ -358,34 +358,35 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
   // Direct-to-LDS source offsets.  Lane l of instruction i lands at LDS i*1024 + l*16, i.e. token
   // t = i*TPI + l/LPT (LPT lanes per token row), 16-byte slot l%LPT of that row.  The chunk fetched into
   // slot s of token t is s ^ f(t), with f chosen per operand so that the MFMA-layout reads are conflict free:
-  //   16-bit, 256-byte rows  K: f = t%16       V: f = 2*(t%8)
+  //   16-bit, 256/512-byte rows  K: f = t%16   V: f = 2*(t%8)      (a 512-byte row: within each 256-byte half)
   //   16-bit, 128-byte rows  K: f = (t/2)%8    V: f = 2*((t/2)%4)
   //   fp8 (128-byte rows)    K: f = (t/2)%8    V: f = (t/2)%4 + 4*((t/16)%2)
   constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
-  // With 256-byte rows the patterns repeat every 4 (K) and 2 (V) instructions; with 128-byte rows every 2 (K), and V
-  // is the same for all (16-bit) or changes once half way (fp8).  A wave keeps one offset register per distinct
-  // pattern among the instructions it issues.
+  // With 256-byte (512-byte) rows the patterns repeat every 4 (8) instructions for K and 2 (4) for V; with 128-byte
+  // rows every 2 (K), and V is the same for all (16-bit) or changes once half way (fp8).  A wave keeps one offset
+  // register per distinct pattern among the instructions it issues.
   const int ts = lane / LPT, slot = lane % LPT;
-  constexpr int NKO = NIW < (ROW128 ? 2 : 4) ? NIW : (ROW128 ? 2 : 4);
-  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < 2 ? NIW : 2));
+  constexpr int PK = ROW128 ? 2 : 16 / G::TPI, PV = 8 / G::TPI;  // pattern periods (PV: wide 16-bit rows only)
+  constexpr int NKO = NIW < PK ? NIW : PK;
+  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < PV ? NIW : PV));
   uint32_t voff_k[NKO], voff_v[NVO];
 #pragma unroll
   for (int e = 0; e < NKO; e++) {
     const int i = i0 + e;
-    voff_k[e] = ts * row_stride + (ROW128 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((4 * i + ts) & 15)) << 4));
+    voff_k[e] = ts * row_stride + (ROW128 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((G::TPI * i + ts) & 15)) << 4));
   }
 #pragma unroll
   for (int e = 0; e < NVO; e++) {
     const int i = FP8 ? (NIW == 4 ? 2 * e : i0) : i0 + e;
     voff_v[e] = ts * row_stride + (FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4)
-                                      : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((4 * i + ts) & 7))) << 4)));
+                                      : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((G::TPI * i + ts) & 7))) << 4)));
   }
   auto k_sel = [](int ii) __attribute__((always_inline)) { return ii % NKO; };
   auto v_sel = [](int ii) __attribute__((always_inline)) { return FP8 ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
   constexpr int NKA = ROW128 ? 2 : 4;
-  uint32_t kaddr[NKA], vaddr[NDB];
+  uint32_t kaddr[NKA], vaddr[NDB < 8 ? NDB : 8];  // (512-byte rows: the second 256 bytes are reached with an immediate)
   if constexpr (R128) {
     // head dim 64: K rows of 128 bytes read exactly like the fp8 K rows (16-byte chunk g + 4j of row c), V^T like the
     // 256-byte-row case with four 32-byte slots per row instead of eight
@@ -396,10 +397,10 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
     for (int db = 0; db < NDB; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 128 + ((tk >> 1) & 3) * 32 + (c & 3) * 8) ^ (db * 32));
   } else if constexpr (!FP8) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) kaddr[j] = lds_wave + (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
+    for (int j = 0; j < 4; j++) kaddr[j] = lds_wave + (uint32_t)(c * G::ROW + (((4 * j + g) ^ c) & 15) * 16);
     const int tk = 4 * g + c / 4;  // transpose read: lane supplies row tk, 8 bytes at column group c%4
 #pragma unroll
-    for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 256 + (tk & 7) * 32 + (c & 3) * 8) ^ (db * 32));
+    for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * G::ROW + (tk & 7) * 32 + (c & 3) * 8) ^ (db * 32));
   } else {
 #pragma unroll
     for (int j = 0; j < 2; j++) kaddr[j] = lds_wave + (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
@@ -574,11 +575,11 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j] + (SOFF + tb * HALF));
+        for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
 #pragma unroll
       for (int db = 0; db < NDB; db++) {
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + SOFF));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db] + (SOFF + HALF)));
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
         u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
         va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
       }
@@ -813,7 +814,7 @@ __global__ __launch_bounds__(NW * 64, SHW > 1 ? 2 : 1) void paged_decode_mfma_ke
         if (LATE) issue_ahead(ring);
         TM(tm_issue)
         moved = run_score_step(ring);
-        if constexpr (SH || (FP8 && NRB == 2)) {
+        if constexpr ((SH && D <= 128) || (FP8 && NRB == 2)) {
           // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
           if (__builtin_expect(moved, 0)) rescale();
           moved = false;
@@ -872,16 +873,17 @@ __global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_
   const int s = r / p.group, gi = r - s * p.group;
   if (p.cu_q && r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
   const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
-  // every lane owns two head elements; with head dim 64 the upper half of the wave idles (reads element 0, stores nothing)
+  // every lane owns two head elements of the 128 this workgroup merges (blockIdx.z picks the half of a 256-wide
+  // head); with head dim 64 the upper half of the wave idles (reads element 0, stores nothing)
   const int hd = p.dim;
   const bool owns = 2 * lane < hd;
-  const int dl = owns ? 2 * lane : 0;
+  const int dl = owns ? 2 * lane + 128 * (int)blockIdx.z : 0;
   uint32_t* op = (uint32_t*)((uint16_t*)p.out + orow * hd) + (dl >> 1);
   auto store = [&](float a0, float a1, float lse) {
     if (!owns) return;
     if (p.final_o) {
       *(f32x2*)(p.final_o + orow * hd + dl) = f32x2{a0, a1};
-      if (lane == 0) p.final_lse[orow] = lse;
+      if (lane == 0 && blockIdx.z == 0) p.final_lse[orow] = lse;
     } else {
       *op = Mma<QT>::pack(a0, a1);
     }
@@ -995,25 +997,27 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   if (skip_combine) return nullptr;
   // four waves per row when sequences span many partitions on average, one otherwise (fewer waves to launch)
   if ((int64_t)p.n_parts > 8 * (int64_t)p.batch)
-    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), dim3(p.heads_kv * p.rows, p.batch), dim3(256), 0, s, p, ws_prefix);
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), dim3(p.heads_kv * p.rows, p.batch, D > 128 ? 2 : 1), dim3(256), 0, s, p, ws_prefix);
   else
-    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), dim3(p.heads_kv * p.rows, p.batch), dim3(64), 0, s, p, ws_prefix);
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), dim3(p.heads_kv * p.rows, p.batch, D > 128 ? 2 : 1), dim3(64), 0, s, p, ws_prefix);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
-// Row blocks (16 query rows each) per wave: one up to 16 rows per kv head, else two.
-int row_blocks_for(int rows) { return rows <= 16 ? 1 : 2; }
+// Row blocks (16 query rows each) per wave: one up to 16 rows per kv head, else two -- one always at head dim 256,
+// where two blocks of accumulators and operands do not fit the register file.
+int row_blocks_for(int rows, int dim) { return (rows <= 16 || dim == 256) ? 1 : 2; }
 
 // Waves per LDS ring.  Up to 32 rows per kv head there is one row group and every wave has its own ring.  Beyond, the
 // 32-row groups of a kv head would each fetch the same K/V tiles: 8, 4 or 2 of them share one ring (a fraction of the
 // fetch instructions per wave, one trip through the memory system per tile); an odd count is rounded up by one idle
 // row group.  Eight waves a compute unit either way (accumulators of two row blocks fit ordinary vector registers);
 // the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
-// (narrow = 128-byte rows, fp8 or head dim 64: four fetch instructions per K tile, so at most four waves share them)
-int ring_waves_for(int rows, bool narrow) {
-  const int n = row_groups(rows, 2);
-  if (rows <= 32) return 1;
+// (narrow = at most four waves to a ring: 128-byte rows, fp8 or head dim 64, have four fetch instructions per K tile;
+// 512-byte rows, head dim 256, keep their accumulators in AGPRs and run one wave per SIMD)
+int ring_waves_for(int rows, int nrb, bool narrow) {
+  const int n = row_groups(rows, nrb);
+  if (n <= 1) return 1;
   const int even = (n + 1) / 2 * 2;
   if (even % 8 == 0 && !narrow) return 8;
   if (even % 4 == 0) return 4;
@@ -1023,14 +1027,17 @@ int ring_waves_for(int rows, bool narrow) {
 template <typename QT, typename KVT, int D>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   constexpr bool SMALL = Geom<KVT, D>::ROW == 128;  // 8 KiB stages: eight unshared waves a CU, four-deep pair rings
-  if (row_blocks_for(p.rows) == 1) return launch_t4<QT, KVT, 1, 2, SMALL ? 8 : 4, 1, D>(p, ws_prefix, skip_combine, s);
-  switch (ring_waves_for(p.rows, SMALL)) {
-    case 1: return launch_t4<QT, KVT, 2, 2, SMALL ? 8 : 4, 1, D>(p, ws_prefix, skip_combine, s);
-    case 2: return launch_t4<QT, KVT, 2, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
-    case 4: return launch_t4<QT, KVT, 2, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
+  constexpr bool WIDE = Geom<KVT, D>::ROW == 512;   // 32 KiB stages, accumulators in AGPRs: one wave per SIMD at most
+  constexpr int NWU = SMALL ? 8 : (WIDE ? 2 : 4);   // unshared waves per workgroup (two stages each fill the LDS)
+  if (p.rows <= 16) return launch_t4<QT, KVT, 1, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
+  constexpr int NRB = WIDE ? 1 : 2;  // == row_blocks_for(rows > 16, D)
+  switch (ring_waves_for(p.rows, NRB, SMALL || WIDE)) {
+    case 1: return launch_t4<QT, KVT, NRB, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
+    case 2: return launch_t4<QT, KVT, NRB, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
+    case 4: return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
     default:
-      if constexpr (!SMALL) return launch_t4<QT, KVT, 2, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
-      return "MFMA kernel: no ring of eight waves with 128-byte rows";
+      if constexpr (!SMALL && !WIDE) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
 
@@ -1041,7 +1048,7 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap) {
   (void)q_len; (void)heads; (void)heads_kv; (void)softcap;
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  if (!(dim == 128 || (dim == 64 && !fp8))) return false;
+  if (!(dim == 128 || ((dim == 64 || dim == 256) && !fp8))) return false;
   if (!(page_size == 16 || page_size % kCT == 0)) return false;
   if (!fp8 && kv_dtype != q_dtype) return false;
   return true;
@@ -1051,11 +1058,11 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
 int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  const int nrb = row_blocks_for(rows), shw = ring_waves_for(rows, fp8 || dim == 64);
+  const int nrb = row_blocks_for(rows, dim), shw = ring_waves_for(rows, nrb, fp8 || dim != 128);
   const int n_rg = ring_row_groups(rows, nrb, shw);
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
-  const int waves_per_cu = (fp8 || dim == 64 || shw > 1) ? 8 : 4;
+  const int waves_per_cu = dim == 256 ? (shw > 1 ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
@@ -1087,6 +1094,11 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
     if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 64>(p, ws_prefix, skip_combine, s);
     if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 64>(p, ws_prefix, skip_combine, s);
     return "MFMA kernel: head dim 64 needs a 16-bit cache of the query's element type";
+  }
+  if (p.dim == 256) {
+    if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 256>(p, ws_prefix, skip_combine, s);
+    if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 256>(p, ws_prefix, skip_combine, s);
+    return "MFMA kernel: head dim 256 needs a 16-bit cache of the query's element type";
   }
   if (p.dim != 128) return "MFMA kernel: unsupported head dim";
   if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 128>(p, ws_prefix, skip_combine, s);

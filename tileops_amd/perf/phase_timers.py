@@ -30,17 +30,18 @@ TIMER_LIB = Path(build_mod.LIB_PATH).with_name("libmi355_tileops_phase_timers.so
 NAMES = ("issue", "wait", "compute", "segment", "prologue", "total")
 
 
-def _row_blocks(rows: int) -> int:
+def _row_blocks(rows: int, dim: int) -> int:
     """Row blocks per wave the launcher picks (csrc/paged_decode_mfma.hip: row_blocks_for)."""
-    return 1 if rows <= 16 else 2
+    return 1 if (rows <= 16 or dim == 256) else 2
 
 
-def _ring_waves(rows: int, fp8: bool) -> int:
+def _ring_waves(rows: int, nrb: int, narrow: bool) -> int:
     """Waves per shared LDS ring (csrc/paged_decode_mfma.hip: ring_waves_for)."""
-    if rows <= 32:
+    n = (rows + 16 * nrb - 1) // (16 * nrb)
+    if n <= 1:
         return 1
-    even = ((rows + 31) // 32 + 1) // 2 * 2
-    if even % 8 == 0 and not fp8:
+    even = (n + 1) // 2 * 2
+    if even % 8 == 0 and not narrow:
         return 8
     return 4 if even % 4 == 0 else 2
 
@@ -56,10 +57,11 @@ def run(name: str, hot: bool = False) -> None:
                                                 inp.block_table.shape[1], inp.q.dtype, inp.k.dtype, 0, native.KERNEL_MFMA)
     fp8 = inp.k.dtype == FP8
     rows = cfg.q_len * (cfg.heads // cfg.heads_kv)
-    nrb, shw = _row_blocks(rows), _ring_waves(rows, fp8)
+    nrb = _row_blocks(rows, cfg.dim)
+    shw = _ring_waves(rows, nrb, fp8 or cfg.dim != 128)
     n_rg = ((rows + 16 * nrb - 1) // (16 * nrb) + shw - 1) // shw * shw  # whole rings
     waves = nparts * cfg.heads_kv * n_rg
-    nw = shw if shw > 1 else (8 if fp8 else 4)  # waves per workgroup
+    nw = shw if shw > 1 else (8 if (fp8 or cfg.dim == 64) else (2 if cfg.dim == 256 else 4))  # waves per workgroup
     if shw > 1:
         waves = shw * 8 * (n_rg // shw) * ((nparts * cfg.heads_kv + 7) // 8)  # grid padded to whole rounds of the 8 XCDs
     ws = torch.zeros(nbytes + waves * 32 + 4096, dtype=torch.uint8, device=dev)
