@@ -1,4 +1,4 @@
-// MFMA paged GQA decode for gfx950 (MI355X): head_dim 128, bf16/fp16 or FP8-e4m3fn KV.
+// MFMA paged GQA decode for gfx950 (MI355X): head dim 128 with bf16/fp16 or FP8-e4m3fn KV, head dims 64 and 256 with bf16/fp16 KV.
 //
 // What it computes is the reference's split kernel + combine
 // (src/tileops/kernels/attention/gqa_decode_paged.py:209-374): per (sequence, kv head), online softmax in

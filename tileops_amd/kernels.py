@@ -281,7 +281,7 @@ class GQADecodePagedKernel(Kernel):
 class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
     """MFMA paged GQA decode on gfx950: direct-to-LDS page gather, QK^T and PV on the matrix cores, the KV
     tile stream partitioned evenly over all compute units.  Serves the region the HIP library reports as
-    supported (head_dim 128, page size a multiple of 16, ...); everything else stays on the general kernel."""
+    supported (head dims 64, 128, 256, page size 16 or a multiple of 32, ...); everything else stays on the general kernel."""
 
     general = False
     _native_kernel = native.KERNEL_MFMA
@@ -405,7 +405,7 @@ class GQADecodeKernel(Kernel):
 class GQADecodeMfmaKernel(GQADecodeKernel):
     """MFMA GQA decode over a contiguous cache: the paged MFMA kernel with identity addressing.  Takes the place of
     the reference's specialised sibling (``GQADecodeBs1Kernel``, src/tileops/kernels/attention/gqa_decode_bs1.py):
-    it states the narrower region it serves (head_dim 128, ...) and wins there, for any batch."""
+    it states the narrower region it serves (head dims 64, 128, 256, ...) and wins there, for any batch."""
 
     general = False
     _native_kernel = native.KERNEL_MFMA
