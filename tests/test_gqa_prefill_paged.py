@@ -307,6 +307,26 @@ def test_llama_shape_chunks_of_hundreds_of_rows_against_long_prefixes(fp8):
     _run(op, case, 64, torch.float16, fp8=fp8)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim, heads, heads_kv", [(256, 16, 4), (64, 16, 2), (256, 8, 8)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_head_dims_64_and_256_with_chunks_of_hundreds_of_rows(dim, heads, heads_kv, dtype):
+    """The reference's qwen3.5 rows use head dim 256 and its softcap rows head dim 64 (attention.yaml:280-289): chunks of
+    hundreds of rows against prefixes spanning several partitions, a chunk that ends mid-page, an empty cache."""
+    require_gfx950()
+    q_lens, old_lens = [257, 96, 40], [1500, 0, 333]
+    case = _case(q_lens, old_lens, heads, heads_kv, dim, dtype, page=64, max_pages=30, seed=23)
+    op = PrefillOp(batch=3, heads=heads, heads_kv=heads_kv, max_pages_per_req=30, page_size=64, dim=dim)
+    _run(op, case, 64, dtype)
+
+
+@pytest.mark.gpu
+def test_fused_rope_head_dim_256_partial_rotary_like_the_qwen_rows():
+    """attention.yaml:280-281 at reduced size: head dim 256, rotary_dim 64, mixed chunk lengths against long prefixes."""
+    require_gfx950()
+    _fused_rope_case([256, 40, 130], [1024, 3000, 7], 16, 4, 256, torch.float16, 64, 3200, True, None, atol=5e-3, max_pages=50)
+
+
 
 @pytest.mark.gpu
 @pytest.mark.parametrize(
