@@ -7,13 +7,14 @@
 //
 //  * Work unit = one wave.  A wave owns (partition, kv head, block of query rows) and runs on its own; only when a
 //    kv head has several blocks of query rows do 2, 4 or 8 such waves share their LDS stages and meet at one
-//    barrier per tile (see the kernel's template parameter SHW).  The KV "tile stream" (every 32-token tile of every sequence, in batch
-//    order) is cut into n_parts equal contiguous ranges computed on the device from real_seqlen_kv, so all
+//    barrier per tile (see the kernel's template parameter SHW).  The KV "tile stream" (every 32-token tile of
+//    every sequence, in batch order) is cut into n_parts equal contiguous ranges computed on the device from
+//    real_seqlen_kv, so all
 //    compute units get the same number of tiles whatever the length distribution, and nothing is read back
 //    to the host.  A range that covers a whole sequence writes the output directly; a range that starts or
 //    ends inside a sequence writes an fp32 partial (at most two per wave) that the combine kernel merges.
 //  * Page gather = 128-bit direct-to-LDS loads (global_load_lds_dwordx4) with the non-temporal hint, 1 KiB
-//    per wave instruction covering whole 256-byte (bf16) or 128-byte (fp8) K/V rows, NS stages per wave in
+//    per wave instruction covering whole 128-, 256- or 512-byte K/V rows (head dim x element size), NS stages per wave in
 //    flight, waited on with s_waitcnt vmcnt.  The LDS image is XOR-swizzled by choosing which 16-byte chunk
 //    each lane fetches, so the reads below are bank-conflict free.
 //  * QK^T: S^T[token][row] = K . Q^T on v_mfma_f32_16x16x32 (K rows straight from LDS as the A operand,
@@ -45,7 +46,9 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // head dim of the fp8 path (16-bit caches also run 64 and 256)
 constexpr int kNumCU = 256;   // MI355X
-constexpr bool kLateIssueFp8 = true;
+// Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
+// landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
+constexpr bool kLateIssueNarrow = true;
 
 // Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
 // hold row groups past the last query row, which load nothing, mask everything and store nothing.
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
   // or after it (a tile lands before the next is requested: fewer requests in flight per compute unit).
-  constexpr bool LATE = SH || (Geom<KVT, D>::ROW == 128 && NRB == 1 && kLateIssueFp8);
+  constexpr bool LATE = SH || (Geom<KVT, D>::ROW == 128 && NRB == 1 && kLateIssueNarrow);
   constexpr int NIW = G::NI / SHW;                     // K (or V) fetch instructions per stage issued by this wave
   constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
