@@ -414,3 +414,50 @@ def _fused_rope_case(q_lens, old_lens, heads, heads_kv, dim, dtype, rotary_dim, 
         for i in range(n):
             touched[physical_pos(table, b, old + i, page)] = True
     assert torch.equal(k_dev[~touched], k_pages[~touched])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rope", [False, True])
+def test_prefill_kernels_capture_into_a_graph_and_replay_on_new_values(rope):
+    """The library calls behind the prefill kernel classes enqueue only (no allocation, no synchronisation, no host read
+    of device data), so a kernel's ``forward`` can be captured in a HIP graph: every replay, with new query and chunk
+    values written into the same tensors, must equal the eager call on the same contents -- output and appended pages."""
+    require_gfx950()
+    from tileops_amd.kernels import GQAPrefillPagedWithKVCacheFwdKernel, GQAPrefillPagedWithKVCacheRopeFwdKernel
+
+    q_lens, old_lens, heads, heads_kv, dim, dtype = [40, 7, 130], [300, 0, 1000], 16, 4, 128, torch.bfloat16
+    case = [t.to(DEV) for t in _case(q_lens, old_lens, heads, heads_kv, dim, dtype, page=64, max_pages=20, seed=51)]
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+    kw = dict(batch=3, heads=heads, heads_kv=heads_kv, max_pages_per_req=20, page_size=64, dim=dim, is_causal=True, dtype=dtype)
+    if rope:
+        kernel = GQAPrefillPagedWithKVCacheRopeFwdKernel(max_position=1200, rotary_dim=64, **kw)
+        cos, sin = (t.to(DEV) for t in rope_tables(64, 1200, 10000.0, dtype))
+        call = lambda: kernel(q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table, max(q_lens), cos, sin)  # noqa: E731
+    else:
+        kernel = GQAPrefillPagedWithKVCacheFwdKernel(**kw)
+        call = lambda: kernel(q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table, max(q_lens))  # noqa: E731
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            call()  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = call()
+    previous = None
+    for it in range(3):
+        if it:
+            q.mul_(-0.75)
+            k_new.mul_(1.0 + 0.5 * it)
+            v_new.add_(0.125 * it)
+        graph.replay()
+        torch.cuda.synchronize()
+        pages_g = (k_pages.clone(), v_pages.clone())
+        eager = call()
+        torch.cuda.synchronize()
+        assert torch.isfinite(eager).all()
+        assert torch.equal(out_g, eager), f"replay {it} differs from the eager call"
+        assert torch.equal(pages_g[0], k_pages) and torch.equal(pages_g[1], v_pages)
+        assert previous is None or not torch.equal(previous, eager)
+        previous = eager.clone()
