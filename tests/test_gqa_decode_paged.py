@@ -188,6 +188,24 @@ def test_ragged_lengths_tails_permuted_tables_and_poison(kernel_key, dtype, fp8,
     _run_and_compare(op, case, 64, tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("page", [16, 32, 64, 128])
+@pytest.mark.parametrize("q_len", [1, 3], ids=["one-row-block", "two-row-blocks"])
+def test_fp8_cache_at_head_dim_64_on_the_mfma_kernel(dtype, page, q_len):
+    """64-byte rows: two fetch instructions per K tile, four lanes per token row, their own LDS swizzles.  Ragged lengths
+    with tails, a length-1 and an empty sequence, permuted pages, NaN in every token that no table addresses."""
+    require_gfx950()
+    lens = [q_len, 0, 63, 64, 65, 777, 2051, 130]
+    case = _ragged_case(len(lens), 32, 4, 64, page, lens, dtype, q_len=q_len, fp8=True, seed=57)
+    if q_len == 1:
+        op = PagedOp(len(lens), 32, 4, case[1].shape[0], 64, page)
+    else:
+        op = MultiOp(len(lens), q_len, 32, 4, case[1].shape[0], 64, page, is_causal=True)
+    assert _serves(op, "gqa_decode_paged_mfma_kernel", dtype, True)
+    _force(op, "gqa_decode_paged_mfma_kernel")
+    _run_and_compare(op, case, page, 3e-2, **({} if q_len == 1 else {"is_causal": True}))
+
+
 def _serves(op, key, dtype, fp8):
     call = op.attention_call(dtype, torch.float8_e4m3fn if fp8 else None, torch.device(DEV, 0))
     return op.kernel_map[key].refusal(call) is None
@@ -266,8 +284,8 @@ def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, 
     end inside sequences, tails shorter than a tile, a sequence shorter than the chunk, NaN in every unaddressed token;
     head counts that leave the grid with workgroups past the last (partition, kv head)."""
     require_gfx950()
-    if fp8 and dim != 128:
-        pytest.skip("the fp8 MFMA path is head dim 128 only")
+    if fp8 and dim == 256:
+        pytest.skip("the fp8 MFMA path serves head dims 64 and 128")
     lens = [2100, q_len, q_len + 33, 700, q_len + 31, q_len + 1]
     case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, dtype, q_len=q_len, fp8=fp8, seed=31)
     op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], dim, 64, is_causal=True)

@@ -1,4 +1,4 @@
-// MFMA paged GQA decode for gfx950 (MI355X): head dim 128 with bf16/fp16 or FP8-e4m3fn KV, head dims 64 and 256 with bf16/fp16 KV.
+// MFMA paged GQA decode for gfx950 (MI355X): head dims 64 and 128 with bf16/fp16 or FP8-e4m3fn KV, head dim 256 with bf16/fp16 KV.
 //
 // What it computes is the reference's split kernel + combine
 // (src/tileops/kernels/attention/gqa_decode_paged.py:209-374): per (sequence, kv head), online softmax in
@@ -44,7 +44,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2;
 #define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
-constexpr int kD = 128;       // head dim of the fp8 path (16-bit caches also run 64 and 256)
+constexpr int kD = 128;       // default head dim (64 also runs; 256 with a 16-bit cache)
 constexpr int kNumCU = 256;   // MI355X
 // Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
@@ -58,8 +58,8 @@ constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT, int D = kD> struct Geom {
   static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
-  static_assert(D == 128 || (!FP8 && (D == 64 || D == 256)), "head dim 128, or 64 / 256 with a 16-bit cache");
-  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 128 (fp8; 16-bit head dim 64), 256 or 512
+  static_assert(D == 64 || D == 128 || (!FP8 && D == 256), "head dim 64 or 128, or 256 with a 16-bit cache");
+  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 64 (fp8 head dim 64), 128 (fp8; 16-bit head dim 64), 256 or 512
   static constexpr int TPI = 1024 / ROW;                   // tokens per direct-to-LDS instruction
   static constexpr int NI = kCT / TPI;                     // instructions per K (or V) stage
   static constexpr int KBYTES = kCT * ROW;
@@ -229,11 +229,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   constexpr int NDB = D / 16;   // 16-wide blocks of the head dim in the output
   constexpr bool ROW128 = G::ROW == 128;        // 128-byte rows: fp8, or 16-bit with head dim 64 (8 KiB stages, eight waves a CU)
   constexpr bool R128 = ROW128 && !FP8;         // 16-bit rows of 128 bytes: the fp8 K layout with 16-bit elements
+  constexpr bool ROW64 = G::ROW == 64;          // fp8 with head dim 64: 4.25 KiB stages, two fetch instructions per K tile
   constexpr bool SH = SHW > 1;
   static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
   // or after it (a tile lands before the next is requested: fewer requests in flight per compute unit).
-  constexpr bool LATE = SH || (Geom<KVT, D>::ROW == 128 && NRB == 1 && kLateIssueNarrow);
+  constexpr bool LATE = SH || (Geom<KVT, D>::ROW <= 128 && NRB == 1 && kLateIssueNarrow);
   constexpr int NIW = G::NI / SHW;                     // K (or V) fetch instructions per stage issued by this wave
   constexpr int IPSW = 2 * NIW + (FP8 ? 1 : 0);        // vector-memory instructions per stage issued by this wave
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -364,31 +365,35 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   //   16-bit, 256/512-byte rows  K: f = t%16   V: f = 2*(t%8)      (a 512-byte row: within each 256-byte half)
   //   16-bit, 128-byte rows  K: f = (t/2)%8    V: f = 2*((t/2)%4)
   //   fp8 (128-byte rows)    K: f = (t/2)%8    V: f = (t/2)%4 + 4*((t/16)%2)
-  constexpr int LPT = G::ROW / 16;  // 16 (bf16) or 8 (fp8)
+  //   fp8 (64-byte rows)     K: f = (t/4)%4    V: f = (t/4)%2 + 2*((t/16)%2)
+  constexpr int LPT = G::ROW / 16;  // lanes per token row: 32, 16, 8 or 4
   // With 256-byte (512-byte) rows the patterns repeat every 4 (8) instructions for K and 2 (4) for V; with 128-byte
-  // rows every 2 (K), and V is the same for all (16-bit) or changes once half way (fp8).  A wave keeps one offset
-  // register per distinct pattern among the instructions it issues.
+  // rows every 2 (K), and V is the same for all (16-bit) or changes once half way (fp8); with 64-byte rows K is the
+  // same for both instructions and V differs between them.  A wave keeps one offset register per distinct pattern
+  // among the instructions it issues.
   const int ts = lane / LPT, slot = lane % LPT;
-  constexpr int PK = ROW128 ? 2 : 16 / G::TPI, PV = 8 / G::TPI;  // pattern periods (PV: wide 16-bit rows only)
+  constexpr int PK = ROW64 ? 1 : (ROW128 ? 2 : 16 / G::TPI), PV = 8 / G::TPI;  // pattern periods (PV: wide 16-bit rows only)
   constexpr int NKO = NIW < PK ? NIW : PK;
-  constexpr int NVO = FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < PV ? NIW : PV));
+  constexpr int NVO = ROW64 ? NIW : (FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < PV ? NIW : PV)));
   uint32_t voff_k[NKO], voff_v[NVO];
 #pragma unroll
   for (int e = 0; e < NKO; e++) {
     const int i = i0 + e;
-    voff_k[e] = ts * row_stride + (ROW128 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((G::TPI * i + ts) & 15)) << 4));
+    voff_k[e] = ts * row_stride + (ROW64 ? ((slot ^ ((ts / 4) & 3)) << 4)
+                                         : (ROW128 ? ((slot ^ ((4 * i + ts / 2) & 7)) << 4) : ((slot ^ ((G::TPI * i + ts) & 15)) << 4)));
   }
 #pragma unroll
   for (int e = 0; e < NVO; e++) {
-    const int i = FP8 ? (NIW == 4 ? 2 * e : i0) : i0 + e;
-    voff_v[e] = ts * row_stride + (FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4)
-                                      : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((G::TPI * i + ts) & 7))) << 4)));
+    const int i = (FP8 && !ROW64) ? (NIW == 4 ? 2 * e : i0) : i0 + e;
+    voff_v[e] = ts * row_stride + (ROW64 ? ((slot ^ (((ts / 4) & 1) + 2 * (i & 1))) << 4)
+                                   : FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4)
+                                         : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((G::TPI * i + ts) & 7))) << 4)));
   }
   auto k_sel = [](int ii) __attribute__((always_inline)) { return ii % NKO; };
-  auto v_sel = [](int ii) __attribute__((always_inline)) { return FP8 ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
+  auto v_sel = [](int ii) __attribute__((always_inline)) { return (FP8 && !ROW64) ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
-  constexpr int NKA = ROW128 ? 2 : 4;
+  constexpr int NKA = ROW64 ? 1 : (ROW128 ? 2 : 4);
   uint32_t kaddr[NKA], vaddr[NDB < 8 ? NDB : 8];  // (512-byte rows: the second 256 bytes are reached with an immediate)
   if constexpr (R128) {
     // head dim 64: K rows of 128 bytes read exactly like the fp8 K rows (16-byte chunk g + 4j of row c), V^T like the
@@ -404,6 +409,14 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
     const int tk = 4 * g + c / 4;  // transpose read: lane supplies row tk, 8 bytes at column group c%4
 #pragma unroll
     for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * G::ROW + (tk & 7) * 32 + (c & 3) * 8) ^ (db * 32));
+  } else if constexpr (ROW64) {
+    // fp8, head dim 64: lane (c, g) reads the 16 bytes of chunk g of token row c, i.e. both 8-wide k-steps of its group
+    kaddr[0] = lds_wave + (uint32_t)(c * 64 + ((g ^ (c >> 2)) & 3) * 16);
+    const int r8 = c >> 1;
+    const int tk = r8 < 4 ? 4 * g + r8 : 16 + 4 * g + (r8 - 4);
+    const int fv = ((tk >> 2) & 1) + 2 * ((tk >> 4) & 1);
+#pragma unroll
+    for (int db = 0; db < NDB; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 64 + fv * 16 + (c & 1) * 8) ^ (db * 16));
   } else {
 #pragma unroll
     for (int j = 0; j < 2; j++) kaddr[j] = lds_wave + (uint32_t)(c * 128 + (((g + 4 * j) ^ (c >> 1)) & 7) * 16);
@@ -565,7 +578,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   // consumes it (widened one 16-column block at a time, in between the MFMAs).
   constexpr bool LATE_V = FP8 && NRB >= 2;
   u32x4 va_op[LATE_V ? 1 : NDB];
-  i32x2 vraw[LATE_V ? 8 : 1];
+  i32x2 vraw[LATE_V ? NDB : 1];
   u32x4 pk[NRB];
   float alpha[NRB];
   auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
@@ -587,29 +600,29 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
       }
     } else {
-      u32x4 kraw[2][2];
-      i32x2 vnow[8];
+      u32x4 kraw[2][NJ / 2];
+      i32x2 vnow[NDB];
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int jj = 0; jj < 2; jj++) kraw[tb][jj] = *LDS_AT(u32x4, kaddr[jj] + (SOFF + tb * 2048));
+        for (int jj = 0; jj < NJ / 2; jj++) kraw[tb][jj] = *LDS_AT(u32x4, kaddr[jj] + (SOFF + tb * HALF));
 #pragma unroll
       for (int tb = 0; tb < 2; tb++) {
         ksc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 64 * tb));
         vsc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 128 + 64 * tb));
       }
 #pragma unroll
-      for (int db = 0; db < 8; db++) vnow[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
+      for (int db = 0; db < NDB; db++) vnow[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int jj = 0; jj < 2; jj++) {
+        for (int jj = 0; jj < NJ / 2; jj++) {
           ka_op[tb][2 * jj] = widen8<QT>(kraw[tb][jj][0], kraw[tb][jj][1]);
           ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
         }
 #pragma unroll
-      for (int db = 0; db < 8; db++) {
+      for (int db = 0; db < NDB; db++) {
         if constexpr (LATE_V) vraw[db] = vnow[db];
         else va_op[db] = widen8<QT>((uint32_t)vnow[db][0], (uint32_t)vnow[db][1]);
       }
@@ -1016,28 +1029,36 @@ int row_blocks_for(int rows, int dim) { return (rows <= 16 || dim == 256) ? 1 : 
 // fetch instructions per wave, one trip through the memory system per tile); an odd count is rounded up by one idle
 // row group.  Eight waves a compute unit either way (accumulators of two row blocks fit ordinary vector registers);
 // the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
-// (narrow = at most four waves to a ring: 128-byte rows, fp8 or head dim 64, have four fetch instructions per K tile;
-// 512-byte rows, head dim 256, keep their accumulators in AGPRs and run one wave per SIMD)
-int ring_waves_for(int rows, int nrb, bool narrow) {
+// (128-byte rows, fp8 or head dim 64, have four fetch instructions per K tile, 64-byte rows two; 512-byte rows, head
+// dim 256, keep their accumulators in AGPRs and run one wave per SIMD)
+int ring_waves_for(int rows, int nrb, int max_ring) {
   const int n = row_groups(rows, nrb);
   if (n <= 1) return 1;
   const int even = (n + 1) / 2 * 2;
-  if (even % 8 == 0 && !narrow) return 8;
-  if (even % 4 == 0) return 4;
+  if (even % 8 == 0 && max_ring >= 8) return 8;
+  if (even % 4 == 0 && max_ring >= 4) return 4;
   return 2;
+}
+// Largest ring for a row width: a ring splits the fetch instructions of a K tile (one per KiB: 8, 4 or 2 for rows of
+// 256, 128 or 64 bytes) evenly over its waves; 512-byte rows stop at four waves, one per SIMD.
+int max_ring_for(int dim, bool fp8) {
+  const int row = dim * (fp8 ? 1 : 2);
+  return row == 256 ? 8 : (row == 64 ? 2 : 4);
 }
 
 template <typename QT, typename KVT, int D>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
-  constexpr bool SMALL = Geom<KVT, D>::ROW == 128;  // 8 KiB stages: eight unshared waves a CU, four-deep pair rings
+  constexpr bool SMALL = Geom<KVT, D>::ROW <= 128;  // 8 KiB stages or less: eight unshared waves a CU, four-deep pair rings
   constexpr bool WIDE = Geom<KVT, D>::ROW == 512;   // 32 KiB stages, accumulators in AGPRs: one wave per SIMD at most
   constexpr int NWU = SMALL ? 8 : (WIDE ? 2 : 4);   // unshared waves per workgroup (two stages each fill the LDS)
   if (p.rows <= 16) return launch_t4<QT, KVT, 1, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
   constexpr int NRB = WIDE ? 1 : 2;  // == row_blocks_for(rows > 16, D)
-  switch (ring_waves_for(p.rows, NRB, SMALL || WIDE)) {
+  switch (ring_waves_for(p.rows, NRB, max_ring_for(D, Geom<KVT, D>::FP8))) {
     case 1: return launch_t4<QT, KVT, NRB, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
     case 2: return launch_t4<QT, KVT, NRB, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
-    case 4: return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
+    case 4:
+      if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
+      return "MFMA kernel: no ring of four waves for this row width";
     default:
       if constexpr (!SMALL && !WIDE) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
@@ -1051,7 +1072,7 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap) {
   (void)q_len; (void)heads; (void)heads_kv; (void)softcap;
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  if (!(dim == 128 || ((dim == 64 || dim == 256) && !fp8))) return false;
+  if (!(dim == 64 || dim == 128 || (dim == 256 && !fp8))) return false;
   if (!(page_size == 16 || page_size % kCT == 0)) return false;
   if (!fp8 && kv_dtype != q_dtype) return false;
   return true;
@@ -1061,7 +1082,7 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
 int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  const int nrb = row_blocks_for(rows, dim), shw = ring_waves_for(rows, nrb, fp8 || dim != 128);
+  const int nrb = row_blocks_for(rows, dim), shw = ring_waves_for(rows, nrb, max_ring_for(dim, fp8));
   const int n_rg = ring_row_groups(rows, nrb, shw);
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
@@ -1096,7 +1117,9 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   if (p.dim == 64) {
     if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 64>(p, ws_prefix, skip_combine, s);
     if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 64>(p, ws_prefix, skip_combine, s);
-    return "MFMA kernel: head dim 64 needs a 16-bit cache of the query's element type";
+    if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag, 64>(p, ws_prefix, skip_combine, s);
+    if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag, 64>(p, ws_prefix, skip_combine, s);
+    return "MFMA kernel: unsupported (q_dtype, kv_dtype) pair";
   }
   if (p.dim == 256) {
     if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 256>(p, ws_prefix, skip_combine, s);

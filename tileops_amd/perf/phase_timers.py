@@ -35,15 +35,16 @@ def _row_blocks(rows: int, dim: int) -> int:
     return 1 if (rows <= 16 or dim == 256) else 2
 
 
-def _ring_waves(rows: int, nrb: int, narrow: bool) -> int:
-    """Waves per shared LDS ring (csrc/paged_decode_mfma.hip: ring_waves_for)."""
+def _ring_waves(rows: int, nrb: int, row_bytes: int) -> int:
+    """Waves per shared LDS ring (csrc/paged_decode_mfma.hip: ring_waves_for, max_ring_for)."""
     n = (rows + 16 * nrb - 1) // (16 * nrb)
     if n <= 1:
         return 1
+    max_ring = 8 if row_bytes == 256 else (2 if row_bytes == 64 else 4)
     even = (n + 1) // 2 * 2
-    if even % 8 == 0 and not narrow:
+    if even % 8 == 0 and max_ring >= 8:
         return 8
-    return 4 if even % 4 == 0 else 2
+    return 4 if (even % 4 == 0 and max_ring >= 4) else 2
 
 
 def run(name: str, hot: bool = False) -> None:
@@ -58,7 +59,7 @@ def run(name: str, hot: bool = False) -> None:
     fp8 = inp.k.dtype == FP8
     rows = cfg.q_len * (cfg.heads // cfg.heads_kv)
     nrb = _row_blocks(rows, cfg.dim)
-    shw = _ring_waves(rows, nrb, fp8 or cfg.dim != 128)
+    shw = _ring_waves(rows, nrb, cfg.dim * (1 if fp8 else 2))
     n_rg = ((rows + 16 * nrb - 1) // (16 * nrb) + shw - 1) // shw * shw  # whole rings
     waves = nparts * cfg.heads_kv * n_rg
     nw = shw if shw > 1 else (8 if (fp8 or cfg.dim == 64) else (2 if cfg.dim == 256 else 4))  # waves per workgroup
