@@ -23,8 +23,10 @@
 //  * PV: O^T[d][row] += V^T . P^T, V^T fetched with LDS transpose reads (ds_read_b64_tr_b16 / _tr_b8).
 //    Query rows sit on the N axis = lane % 16, so every per-row softmax quantity (max, sum, rescale factor)
 //    is lane-local; the only cross-lane traffic is a two-step max/sum over the four 16-lane groups.
-//  * FP8: bytes are widened to bf16/fp16 on the LDS->register path (v_cvt_scalef32_pk_*_fp8, OCP e4m3fn);
-//    the per-token K scale multiplies the score and the V scale multiplies the probability, so no
+//  * FP8: V bytes are widened to bf16/fp16 on the LDS->register path (v_cvt_scalef32_pk_*_fp8, OCP e4m3fn).  At head
+//    dim 128 the K bytes are not widened at all: Q.K^T runs on v_mfma_f32_16x16x128_f8f6f4 against the query row
+//    split into two e4m3fn rows (hi + lo, exact for bf16 queries); at head dim 64 K is widened like V.
+//    The per-token K scale multiplies the score and the V scale multiplies the probability, so no
 //    head_dim-wide multiplies are spent on dequantisation.  Scales ride the same direct-to-LDS pipeline.
 #include "common.h"
 #include "device_utils.h"
@@ -39,6 +41,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 #define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
@@ -93,6 +96,20 @@ template <> struct Mma<fp16_tag> {
     return __builtin_bit_cast(uint32_t, r);
   }
 };
+
+// 16x16 tile of 128-deep dot products of e4m3fn bytes (v_mfma_f32_16x16x128_f8f6f4, no block scales): lane (c, g)
+// supplies 32 bytes of row c of each operand.  Which 32 of the 128 depth positions those are is the same function of g
+// for both operands, so any split of a row into four 32-byte parts may be used as long as both sides use the same.
+__device__ __forceinline__ f32x4 mma_fp8_k128(u32x4 a_lo, u32x4 a_hi, u32x4 b_lo, u32x4 b_hi, f32x4 acc) {
+  i32x8 a = {(int)a_lo[0], (int)a_lo[1], (int)a_lo[2], (int)a_lo[3], (int)a_hi[0], (int)a_hi[1], (int)a_hi[2], (int)a_hi[3]};
+  i32x8 b = {(int)b_lo[0], (int)b_lo[1], (int)b_lo[2], (int)b_lo[3], (int)b_hi[0], (int)b_hi[1], (int)b_hi[2], (int)b_hi[3]};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+}
+// Four floats -> four e4m3fn bytes (round to nearest even; callers keep |x| <= 448).
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+}
 
 // 8 fp8 bytes (two dwords) -> 8 16-bit elements (four dwords), element order preserved.
 template <typename QT> __device__ __forceinline__ u32x4 widen8(uint32_t w0, uint32_t w1) {
@@ -230,6 +247,11 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   constexpr bool ROW128 = G::ROW == 128;        // 128-byte rows: fp8, or 16-bit with head dim 64 (8 KiB stages, eight waves a CU)
   constexpr bool R128 = ROW128 && !FP8;         // 16-bit rows of 128 bytes: the fp8 K layout with 16-bit elements
   constexpr bool ROW64 = G::ROW == 64;          // fp8 with head dim 64: 4.25 KiB stages, two fetch instructions per K tile
+  // Q.K^T on the fp8 matrix instruction (head dim 128 = one 128-deep step): the K bytes go in as they are, the query
+  // row goes in as two e4m3fn rows hi + lo (hi = the row times a power of two, rounded; lo = what the rounding dropped,
+  // rounded again: exact for bf16 queries, within 2^-8 of every fp16 element) and the power of two multiplies the
+  // softmax exponent.
+  constexpr bool QK8 = FP8 && D == 128;
   constexpr bool SH = SHW > 1;
   static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
@@ -528,7 +550,8 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   int limit[NRB];
   const int qoff = (p.causal && p.q_len > 1) ? p.q_len - 1 : 0;
   const bool softcap = p.softcap > 0.f;
-  const uint32_t q_sign = p.negate_q ? 0x80008000u : 0u;
+  const uint32_t q_sign = p.negate_q ? (QK8 ? 0x80808080u : 0x80008000u) : 0u;
+  float q_scale[NRB];  // QK8: the power of two taken out of the lane's query row (row c of each row block)
 
   int seg_q_len = p.q_len;   // query tokens of the sequence being processed (varies with packed queries)
   int64_t seg_q_row0 = 0;    // its first row in q / out
@@ -541,12 +564,48 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       bool valid = r < seg_q_len * p.group;
       int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
       const char* qp = (const char*)p.q + (((seg_q_row0 + s) * p.heads + kvh * p.group + gi) * D) * 2;
+      if constexpr (QK8) {
+        // the lane's 32 depth positions are those of the K bytes it reads: head elements [16g, 16g+16) and [64+16g, 64+16g+16)
+        float f[32];
 #pragma unroll
-      for (int j = 0; j < NJ; j++) {
-        // head elements this lane contributes to k-step j: 8 consecutive ones, matching the K operand
-        int d0 = FP8 ? 64 * (j >> 1) + 16 * g + 8 * (j & 1) : 32 * j + 8 * g;
-        u32x4 z = {0, 0, 0, 0};
-        qreg[rb][j] = valid ? *(const u32x4*)(qp + d0 * 2) : z;
+        for (int h = 0; h < 4; h++) {
+          u32x4 z = {0, 0, 0, 0};
+          u32x4 raw = valid ? *(const u32x4*)(qp + (64 * (h >> 1) + 16 * g + 8 * (h & 1)) * 2) : z;
+          uint32_t w[4] = {raw[0], raw[1], raw[2], raw[3]};
+          Unpack<QT, 8>::run(w, f + 8 * h);
+        }
+        float am = 0.f;
+#pragma unroll
+        for (int e = 0; e < 32; e++) am = fmaxf(am, fabsf(f[e]));
+        am = fmaxf(group_max(am), 1e-30f);  // over the four lanes that share the row
+        // scale by a power of two that puts the row maximum in [128, 256): element mantissas are untouched, so the
+        // eight significant bits of a bf16 element are exactly hi (four) + lo (four)
+        const uint32_t be = (__float_as_uint(am) >> 23) & 0xffu;  // biased exponent, >= 27
+        const float inv = __uint_as_float((261u - be) << 23);     // 2^(7 - e)
+        q_scale[rb] = __uint_as_float((be - 7u) << 23);            // 2^(e - 7)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {   // h = which 16 of the lane's 32 positions
+          u32x4 hi, lo;
+#pragma unroll
+          for (int w4 = 0; w4 < 4; w4++) {
+            const float* x = f + 16 * h + 4 * w4;
+            const float a0 = x[0] * inv, a1 = x[1] * inv, a2 = x[2] * inv, a3 = x[3] * inv;
+            const uint32_t wh = pack_fp8x4(a0, a1, a2, a3);
+            const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(wh, false), b23 = __builtin_amdgcn_cvt_pk_f32_fp8(wh, true);
+            hi[w4] = wh;
+            lo[w4] = pack_fp8x4(a0 - b01[0], a1 - b01[1], a2 - b23[0], a3 - b23[1]);
+          }
+          qreg[rb][h] = hi;      // [0], [1]: hi part, the lane's 32 bytes
+          qreg[rb][2 + h] = lo;  // [2], [3]: lo part
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          // head elements this lane contributes to k-step j: 8 consecutive ones, matching the K operand
+          int d0 = FP8 ? 64 * (j >> 1) + 16 * g + 8 * (j & 1) : 32 * j + 8 * g;
+          u32x4 z = {0, 0, 0, 0};
+          qreg[rb][j] = valid ? *(const u32x4*)(qp + d0 * 2) : z;
+        }
       }
       limit[rb] = valid ? ((p.causal && p.q_len > 1) ? cu.len - seg_q_len + s + 1 : cu.len) : 0;
       m_run[rb] = kNegFloor;
@@ -618,8 +677,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
         for (int jj = 0; jj < NJ / 2; jj++) {
-          ka_op[tb][2 * jj] = widen8<QT>(kraw[tb][jj][0], kraw[tb][jj][1]);
-          ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
+          if constexpr (QK8) {  // kept as bytes: [0] = chunk g, [1] = chunk g + 4 of the token row
+            ka_op[tb][jj] = kraw[tb][jj];
+          } else {
+            ka_op[tb][2 * jj] = widen8<QT>(kraw[tb][jj][0], kraw[tb][jj][1]);
+            ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
+          }
         }
 #pragma unroll
       for (int db = 0; db < NDB; db++) {
@@ -634,20 +697,34 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
     for (int tb = 0; tb < 2; tb++)
 #pragma unroll
       for (int rb = 0; rb < NRB; rb++) s_acc[tb][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (QK8) {
 #pragma unroll
-    for (int j = 0; j < NJ; j++)
+      for (int part = 0; part < 2; part++)  // hi, then lo: dependent instructions are 2*NRB apart
 #pragma unroll
-      for (int rb = 0; rb < NRB; rb++)
+        for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
-        for (int tb = 0; tb < 2; tb++) {
-          s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
-        }
+          for (int tb = 0; tb < 2; tb++)
+            s_acc[tb][rb] = mma_fp8_k128(ka_op[tb][0], ka_op[tb][1], qreg[rb][2 * part], qreg[rb][2 * part + 1], s_acc[tb][rb]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+          for (int tb = 0; tb < 2; tb++) {
+            s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
+          }
+    }
     // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
     const bool need_mask = tok0 + kCT > cu.len - qoff;
-    const float exp_scale = softcap ? 1.0f : p.score_scale;
+    const float exp_scale_all = softcap ? 1.0f : p.score_scale;
     bool any_moved = false;
 #pragma unroll
     for (int rb = 0; rb < NRB; rb++) {
+      // QK8: the scores are those of the query row scaled to absmax 448; its scale goes where the softmax scale goes
+      // (kept a positive normal number, so that a masked -inf stays -inf)
+      const float exp_scale = QK8 ? (softcap ? 1.0f : fmaxf(exp_scale_all * q_scale[rb], 1e-37f)) : exp_scale_all;
+      const float inv_cap_scale = QK8 ? p.inv_cap_scale * q_scale[rb] : p.inv_cap_scale;
       float x[2][4];
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
@@ -664,7 +741,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
 #pragma unroll
         for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-          for (int i = 0; i < 4; i++) x[tb][i] = to_logit2<true>(x[tb][i], p.score_scale, p.cap_log2e, p.inv_cap_scale);
+          for (int i = 0; i < 4; i++) x[tb][i] = to_logit2<true>(x[tb][i], p.score_scale, p.cap_log2e, inv_cap_scale);
       }
       if (need_mask) {  // only the last tile(s) of a sequence
 #pragma unroll
