@@ -191,16 +191,18 @@ def test_ragged_lengths_tails_permuted_tables_and_poison(kernel_key, dtype, fp8,
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("page", [16, 32, 64, 128])
 @pytest.mark.parametrize("q_len", [1, 3], ids=["one-row-block", "two-row-blocks"])
-def test_fp8_cache_at_head_dim_64_on_the_mfma_kernel(dtype, page, q_len):
-    """64-byte rows: two fetch instructions per K tile, four lanes per token row, their own LDS swizzles.  Ragged lengths
-    with tails, a length-1 and an empty sequence, permuted pages, NaN in every token that no table addresses."""
+@pytest.mark.parametrize("dim", [64, 256])
+def test_fp8_cache_at_head_dims_64_and_256_on_the_mfma_kernel(dtype, page, q_len, dim):
+    """64-byte rows: two fetch instructions per K tile, four lanes per token row; 256-byte rows: eight instructions, two
+    128-deep score steps, sixteen V^T column blocks; each width with its own LDS swizzles.  Ragged lengths with tails, a
+    length-1 and an empty sequence, permuted pages, NaN in every token that no table addresses."""
     require_gfx950()
     lens = [q_len, 0, 63, 64, 65, 777, 2051, 130]
-    case = _ragged_case(len(lens), 32, 4, 64, page, lens, dtype, q_len=q_len, fp8=True, seed=57)
+    case = _ragged_case(len(lens), 32, 4, dim, page, lens, dtype, q_len=q_len, fp8=True, seed=57)
     if q_len == 1:
-        op = PagedOp(len(lens), 32, 4, case[1].shape[0], 64, page)
+        op = PagedOp(len(lens), 32, 4, case[1].shape[0], dim, page)
     else:
-        op = MultiOp(len(lens), q_len, 32, 4, case[1].shape[0], 64, page, is_causal=True)
+        op = MultiOp(len(lens), q_len, 32, 4, case[1].shape[0], dim, page, is_causal=True)
     assert _serves(op, "gqa_decode_paged_mfma_kernel", dtype, True)
     _force(op, "gqa_decode_paged_mfma_kernel")
     _run_and_compare(op, case, page, 3e-2, **({} if q_len == 1 else {"is_causal": True}))
@@ -284,8 +286,6 @@ def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, 
     end inside sequences, tails shorter than a tile, a sequence shorter than the chunk, NaN in every unaddressed token;
     head counts that leave the grid with workgroups past the last (partition, kv head)."""
     require_gfx950()
-    if fp8 and dim == 256:
-        pytest.skip("the fp8 MFMA path serves head dims 64 and 128")
     lens = [2100, q_len, q_len + 33, 700, q_len + 31, q_len + 1]
     case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, dtype, q_len=q_len, fp8=fp8, seed=31)
     op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], dim, 64, is_causal=True)

@@ -156,12 +156,13 @@ def test_selection_regions():
     mfma_serves = GQADecodePagedMfmaKernel.applies(_call())
     assert key == ("gqa_decode_paged_mfma_kernel" if mfma_serves else "gqa_decode_paged_kernel")
     # shapes outside the specialised region stay on the general kernel
-    for kw in (dict(page_size=24), dict(dim=256, kv_dtype=torch.float8_e4m3fn), dict(dim=96)):
+    for kw in (dict(page_size=24), dict(dim=96), dict(dim=32, kv_dtype=torch.float8_e4m3fn)):
         assert not GQADecodePagedMfmaKernel.applies(_call(**kw))
         assert op.select_kernel_key(PAGED_DECODE_KEYS, _call(**kw)) == "gqa_decode_paged_kernel"
-    # head dims 64 (either cache) and 256 (16-bit cache) are inside it
+    # head dims 64 and 256 are inside it, with either cache
     assert GQADecodePagedMfmaKernel.applies(_call(dim=64)) == mfma_serves
     assert GQADecodePagedMfmaKernel.applies(_call(dim=64, kv_dtype=torch.float8_e4m3fn)) == mfma_serves
+    assert GQADecodePagedMfmaKernel.applies(_call(dim=256, kv_dtype=torch.float8_e4m3fn)) == mfma_serves
     assert GQADecodePagedMfmaKernel.applies(_call(dim=256)) == mfma_serves
     with pytest.raises(ValueError, match="no implementation serves this call"):
         op.select_kernel_key(PAGED_DECODE_KEYS, _call(arch=90))

@@ -1,4 +1,4 @@
-// MFMA paged GQA decode for gfx950 (MI355X): head dims 64 and 128 with bf16/fp16 or FP8-e4m3fn KV, head dim 256 with bf16/fp16 KV.
+// MFMA paged GQA decode for gfx950 (MI355X): head dims 64, 128 and 256 with bf16/fp16 or FP8-e4m3fn KV.
 //
 // What it computes is the reference's split kernel + combine
 // (src/tileops/kernels/attention/gqa_decode_paged.py:209-374): per (sequence, kv head), online softmax in
@@ -24,8 +24,8 @@
 //    Query rows sit on the N axis = lane % 16, so every per-row softmax quantity (max, sum, rescale factor)
 //    is lane-local; the only cross-lane traffic is a two-step max/sum over the four 16-lane groups.
 //  * FP8: V bytes are widened to bf16/fp16 on the LDS->register path (v_cvt_scalef32_pk_*_fp8, OCP e4m3fn).  At head
-//    dim 128 the K bytes are not widened at all: Q.K^T runs on v_mfma_f32_16x16x128_f8f6f4 against the query row
-//    split into two e4m3fn rows (hi + lo, exact for bf16 queries); at head dim 64 K is widened like V.
+//    dims 128 and 256 the K bytes are not widened at all: Q.K^T runs on v_mfma_f32_16x16x128_f8f6f4 against the query
+//    row split into two e4m3fn rows (hi + lo, exact for bf16 queries); at head dim 64 K is widened like V.
 //    The per-token K scale multiplies the score and the V scale multiplies the probability, so no
 //    head_dim-wide multiplies are spent on dequantisation.  Scales ride the same direct-to-LDS pipeline.
 #include "common.h"
@@ -47,7 +47,7 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 #define LDS_AT(T, addr) ((__attribute__((address_space(3))) T*)(uintptr_t)(addr))
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
-constexpr int kD = 128;       // default head dim (64 also runs; 256 with a 16-bit cache)
+constexpr int kD = 128;       // default head dim (64 and 256 also run)
 constexpr int kNumCU = 256;   // MI355X
 // Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
@@ -61,8 +61,8 @@ constexpr float kRescaleGap = 8.0f;  // see the lazy rescale in the softmax step
 
 template <typename KVT, int D = kD> struct Geom {
   static constexpr bool FP8 = ElemTraits<KVT>::bytes == 1;
-  static_assert(D == 64 || D == 128 || (!FP8 && D == 256), "head dim 64 or 128, or 256 with a 16-bit cache");
-  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 64 (fp8 head dim 64), 128 (fp8; 16-bit head dim 64), 256 or 512
+  static_assert(D == 64 || D == 128 || D == 256, "head dim 64, 128 or 256");
+  static constexpr int ROW = D * ElemTraits<KVT>::bytes;   // bytes of one (token, kv head) row: 64, 128 or 256 (fp8), 128, 256 or 512 (16-bit)
   static constexpr int TPI = 1024 / ROW;                   // tokens per direct-to-LDS instruction
   static constexpr int NI = kCT / TPI;                     // instructions per K (or V) stage
   static constexpr int KBYTES = kCT * ROW;
@@ -247,11 +247,13 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   constexpr bool ROW128 = G::ROW == 128;        // 128-byte rows: fp8, or 16-bit with head dim 64 (8 KiB stages, eight waves a CU)
   constexpr bool R128 = ROW128 && !FP8;         // 16-bit rows of 128 bytes: the fp8 K layout with 16-bit elements
   constexpr bool ROW64 = G::ROW == 64;          // fp8 with head dim 64: 4.25 KiB stages, two fetch instructions per K tile
-  // Q.K^T on the fp8 matrix instruction (head dim 128 = one 128-deep step): the K bytes go in as they are, the query
+  constexpr bool F256 = FP8 && G::ROW == 256;   // fp8 with head dim 256: the 16-bit K layout of 256-byte rows, its own V^T layout
+  // Q.K^T on the fp8 matrix instruction (one 128-deep step per 128 head elements): the K bytes go in as they are, the query
   // row goes in as two e4m3fn rows hi + lo (hi = the row times a power of two, rounded; lo = what the rounding dropped,
   // rounded again: exact for bf16 queries, within 2^-8 of every fp16 element) and the power of two multiplies the
   // softmax exponent.
-  constexpr bool QK8 = FP8 && D == 128;
+  constexpr bool QK8 = FP8 && D >= 128;
+  constexpr int NCH = D / 64;  // QK8: 16-byte chunks of a row per lane (chunk j = head elements [64j + 16g, 64j + 16g + 16))
   constexpr bool SH = SHW > 1;
   static_assert(!SH || (NW == SHW && G::NI % SHW == 0), "a shared-stage workgroup is the SHW waves of one ring");
   // Where the next fetch goes out: ahead of the wait for the current tile (one more stage in flight while waiting),
@@ -388,6 +390,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   //   16-bit, 128-byte rows  K: f = (t/2)%8    V: f = 2*((t/2)%4)
   //   fp8 (128-byte rows)    K: f = (t/2)%8    V: f = (t/2)%4 + 4*((t/16)%2)
   //   fp8 (64-byte rows)     K: f = (t/4)%4    V: f = (t/4)%2 + 2*((t/16)%2)
+  //   fp8 (256-byte rows)    K: f = t%16       V: f = t%8 + 8*((t/16)%2)
   constexpr int LPT = G::ROW / 16;  // lanes per token row: 32, 16, 8 or 4
   // With 256-byte (512-byte) rows the patterns repeat every 4 (8) instructions for K and 2 (4) for V; with 128-byte
   // rows every 2 (K), and V is the same for all (16-bit) or changes once half way (fp8); with 64-byte rows K is the
@@ -396,7 +399,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   const int ts = lane / LPT, slot = lane % LPT;
   constexpr int PK = ROW64 ? 1 : (ROW128 ? 2 : 16 / G::TPI), PV = 8 / G::TPI;  // pattern periods (PV: wide 16-bit rows only)
   constexpr int NKO = NIW < PK ? NIW : PK;
-  constexpr int NVO = ROW64 ? NIW : (FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < PV ? NIW : PV)));
+  constexpr int NVO = F256 ? (NIW == 8 ? 4 : 2) : ROW64 ? NIW : (FP8 ? (NIW == 4 ? 2 : 1) : (R128 ? 1 : (NIW < PV ? NIW : PV)));
   uint32_t voff_k[NKO], voff_v[NVO];
 #pragma unroll
   for (int e = 0; e < NKO; e++) {
@@ -406,17 +409,21 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   }
 #pragma unroll
   for (int e = 0; e < NVO; e++) {
-    const int i = (FP8 && !ROW64) ? (NIW == 4 ? 2 * e : i0) : i0 + e;
-    voff_v[e] = ts * row_stride + (ROW64 ? ((slot ^ (((ts / 4) & 1) + 2 * (i & 1))) << 4)
+    const int i = F256 ? (NIW == 8 ? (e & 1) + 4 * (e >> 1) : i0 + e) : (FP8 && !ROW64) ? (NIW == 4 ? 2 * e : i0) : i0 + e;
+    voff_v[e] = ts * row_stride + (F256 ? ((slot ^ (((4 * i + ts) & 7) + 8 * ((i >> 2) & 1))) << 4)
+                                   : ROW64 ? ((slot ^ (((ts / 4) & 1) + 2 * (i & 1))) << 4)
                                    : FP8 ? ((slot ^ (((ts / 2) & 3) + 4 * ((i >> 1) & 1))) << 4)
                                          : (R128 ? ((slot ^ (2 * ((ts / 2) & 3))) << 4) : ((slot ^ (2 * ((G::TPI * i + ts) & 7))) << 4)));
   }
   auto k_sel = [](int ii) __attribute__((always_inline)) { return ii % NKO; };
-  auto v_sel = [](int ii) __attribute__((always_inline)) { return (FP8 && !ROW64) ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO; };
+  auto v_sel = [](int ii) __attribute__((always_inline)) {
+    if (F256) return NIW == 8 ? (ii & 1) + 2 * ((ii >> 2) & 1) : ii % NVO;
+    return (FP8 && !ROW64) ? (NIW == 4 ? (ii >> 1) & 1 : 0) : ii % NVO;
+  };
 
   // Absolute LDS read addresses of stage slot 0; slot s and token block tb are added as immediates.
   constexpr int NKA = ROW64 ? 1 : (ROW128 ? 2 : 4);
-  uint32_t kaddr[NKA], vaddr[NDB < 8 ? NDB : 8];  // (512-byte rows: the second 256 bytes are reached with an immediate)
+  uint32_t kaddr[NKA], vaddr[F256 ? 16 : (NDB < 8 ? NDB : 8)];  // (512-byte rows: the second 256 bytes are reached with an immediate)
   if constexpr (R128) {
     // head dim 64: K rows of 128 bytes read exactly like the fp8 K rows (16-byte chunk g + 4j of row c), V^T like the
     // 256-byte-row case with four 32-byte slots per row instead of eight
@@ -431,6 +438,16 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
     const int tk = 4 * g + c / 4;  // transpose read: lane supplies row tk, 8 bytes at column group c%4
 #pragma unroll
     for (int db = 0; db < 8; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * G::ROW + (tk & 7) * 32 + (c & 3) * 8) ^ (db * 32));
+  } else if constexpr (F256) {
+    // fp8, head dim 256: K chunks 4j + g of token row c as for 16-bit rows of this width; V^T bytes of sixteen rows per
+    // half wave, one 16-byte chunk each, spread over all banks by f = t%8 + 8*((t/16)%2)
+#pragma unroll
+    for (int j = 0; j < 4; j++) kaddr[j] = lds_wave + (uint32_t)(c * 256 + (((4 * j + g) ^ c) & 15) * 16);
+    const int r8 = c >> 1;
+    const int tk = r8 < 4 ? 4 * g + r8 : 16 + 4 * g + (r8 - 4);
+    const int fv = (tk & 7) + 8 * ((tk >> 4) & 1);
+#pragma unroll
+    for (int db = 0; db < 16; db++) vaddr[db] = lds_wave + G::KBYTES + (uint32_t)((tk * 256 + fv * 16 + (c & 1) * 8) ^ (db * 16));
   } else if constexpr (ROW64) {
     // fp8, head dim 64: lane (c, g) reads the 16 bytes of chunk g of token row c, i.e. both 8-wide k-steps of its group
     kaddr[0] = lds_wave + (uint32_t)(c * 64 + ((g ^ (c >> 2)) & 3) * 16);
@@ -565,10 +582,10 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
       const char* qp = (const char*)p.q + (((seg_q_row0 + s) * p.heads + kvh * p.group + gi) * D) * 2;
       if constexpr (QK8) {
-        // the lane's 32 depth positions are those of the K bytes it reads: head elements [16g, 16g+16) and [64+16g, 64+16g+16)
-        float f[32];
+        // the lane's depth positions are those of the K bytes it reads: head elements [64j + 16g, 64j + 16g + 16), j < NCH
+        float f[16 * NCH];
 #pragma unroll
-        for (int h = 0; h < 4; h++) {
+        for (int h = 0; h < 2 * NCH; h++) {
           u32x4 z = {0, 0, 0, 0};
           u32x4 raw = valid ? *(const u32x4*)(qp + (64 * (h >> 1) + 16 * g + 8 * (h & 1)) * 2) : z;
           uint32_t w[4] = {raw[0], raw[1], raw[2], raw[3]};
@@ -576,7 +593,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         }
         float am = 0.f;
 #pragma unroll
-        for (int e = 0; e < 32; e++) am = fmaxf(am, fabsf(f[e]));
+        for (int e = 0; e < 16 * NCH; e++) am = fmaxf(am, fabsf(f[e]));
         am = fmaxf(group_max(am), 1e-30f);  // over the four lanes that share the row
         // scale by a power of two that puts the row maximum in [128, 256): element mantissas are untouched, so the
         // eight significant bits of a bf16 element are exactly hi (four) + lo (four)
@@ -584,7 +601,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         const float inv = __uint_as_float((261u - be) << 23);     // 2^(7 - e)
         q_scale[rb] = __uint_as_float((be - 7u) << 23);            // 2^(e - 7)
 #pragma unroll
-        for (int h = 0; h < 2; h++) {   // h = which 16 of the lane's 32 positions
+        for (int h = 0; h < NCH; h++) {   // h = which 16 of the lane's positions
           u32x4 hi, lo;
 #pragma unroll
           for (int w4 = 0; w4 < 4; w4++) {
@@ -595,8 +612,8 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
             hi[w4] = wh;
             lo[w4] = pack_fp8x4(a0 - b01[0], a1 - b01[1], a2 - b23[0], a3 - b23[1]);
           }
-          qreg[rb][h] = hi;      // [0], [1]: hi part, the lane's 32 bytes
-          qreg[rb][2 + h] = lo;  // [2], [3]: lo part
+          qreg[rb][h] = hi;        // [0, NCH): hi part
+          qreg[rb][NCH + h] = lo;  // [NCH, 2 NCH): lo part
         }
       } else {
 #pragma unroll
@@ -635,7 +652,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   // address, and a rescale inside the loop makes the register allocator shuttle all of them on every iteration.
   // With an fp8 cache and several row blocks registers are short: V^T then stays in bytes until the PV product
   // consumes it (widened one 16-column block at a time, in between the MFMAs).
-  constexpr bool LATE_V = FP8 && NRB >= 2;
+  constexpr bool LATE_V = FP8 && (NRB >= 2 || D == 256);
   u32x4 va_op[LATE_V ? 1 : NDB];
   i32x2 vraw[LATE_V ? NDB : 1];
   u32x4 pk[NRB];
@@ -677,7 +694,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
         for (int jj = 0; jj < NJ / 2; jj++) {
-          if constexpr (QK8) {  // kept as bytes: [0] = chunk g, [1] = chunk g + 4 of the token row
+          if constexpr (QK8) {  // kept as bytes: [jj] = chunk 4 jj + g of the token row
             ka_op[tb][jj] = kraw[tb][jj];
           } else {
             ka_op[tb][2 * jj] = widen8<QT>(kraw[tb][jj][0], kraw[tb][jj][1]);
@@ -701,10 +718,13 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
 #pragma unroll
       for (int part = 0; part < 2; part++)  // hi, then lo: dependent instructions are 2*NRB apart
 #pragma unroll
-        for (int rb = 0; rb < NRB; rb++)
+        for (int h = 0; h < NCH / 2; h++)   // 128 head elements per step
 #pragma unroll
-          for (int tb = 0; tb < 2; tb++)
-            s_acc[tb][rb] = mma_fp8_k128(ka_op[tb][0], ka_op[tb][1], qreg[rb][2 * part], qreg[rb][2 * part + 1], s_acc[tb][rb]);
+          for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++)
+              s_acc[tb][rb] = mma_fp8_k128(ka_op[tb][2 * h], ka_op[tb][2 * h + 1], qreg[rb][part * NCH + 2 * h],
+                                           qreg[rb][part * NCH + 2 * h + 1], s_acc[tb][rb]);
     } else {
 #pragma unroll
       for (int j = 0; j < NJ; j++)
@@ -1117,10 +1137,10 @@ int ring_waves_for(int rows, int nrb, int max_ring) {
   return 2;
 }
 // Largest ring for a row width: a ring splits the fetch instructions of a K tile (one per KiB: 8, 4 or 2 for rows of
-// 256, 128 or 64 bytes) evenly over its waves; 512-byte rows stop at four waves, one per SIMD.
+// 256, 128 or 64 bytes) evenly over its waves; head dim 256 stops at four waves, one per SIMD.
 int max_ring_for(int dim, bool fp8) {
   const int row = dim * (fp8 ? 1 : 2);
-  return row == 256 ? 8 : (row == 64 ? 2 : 4);
+  return (row == 256 && dim != 256) ? 8 : (row == 64 ? 2 : 4);
 }
 
 template <typename QT, typename KVT, int D>
@@ -1129,7 +1149,7 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   constexpr bool WIDE = Geom<KVT, D>::ROW == 512;   // 32 KiB stages, accumulators in AGPRs: one wave per SIMD at most
   constexpr int NWU = SMALL ? 8 : (WIDE ? 2 : 4);   // unshared waves per workgroup (two stages each fill the LDS)
   if (p.rows <= 16) return launch_t4<QT, KVT, 1, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
-  constexpr int NRB = WIDE ? 1 : 2;  // == row_blocks_for(rows > 16, D)
+  constexpr int NRB = D == 256 ? 1 : 2;  // == row_blocks_for(rows > 16, D)
   switch (ring_waves_for(p.rows, NRB, max_ring_for(D, Geom<KVT, D>::FP8))) {
     case 1: return launch_t4<QT, KVT, NRB, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
     case 2: return launch_t4<QT, KVT, NRB, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
@@ -1137,7 +1157,7 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
       if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of four waves for this row width";
     default:
-      if constexpr (!SMALL && !WIDE) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      if constexpr (!SMALL && D != 256) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
@@ -1149,7 +1169,7 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap) {
   (void)q_len; (void)heads; (void)heads_kv; (void)softcap;
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
-  if (!(dim == 64 || dim == 128 || (dim == 256 && !fp8))) return false;
+  if (!(dim == 64 || dim == 128 || dim == 256)) return false;
   if (!(page_size == 16 || page_size % kCT == 0)) return false;
   if (!fp8 && kv_dtype != q_dtype) return false;
   return true;
@@ -1163,7 +1183,7 @@ int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   const int n_rg = ring_row_groups(rows, nrb, shw);
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
-  const int waves_per_cu = dim == 256 ? (shw > 1 ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
+  const int waves_per_cu = dim == 256 ? ((shw > 1 || fp8) ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
   const int64_t waves = (int64_t)kNumCU * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
@@ -1201,7 +1221,9 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   if (p.dim == 256) {
     if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 256>(p, ws_prefix, skip_combine, s);
     if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP16) return launch_t2<fp16_tag, fp16_tag, 256>(p, ws_prefix, skip_combine, s);
-    return "MFMA kernel: head dim 256 needs a 16-bit cache of the query's element type";
+    if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<bf16_tag, fp8_tag, 256>(p, ws_prefix, skip_combine, s);
+    if (q_dtype == MI355_DT_FP16 && kv_dtype == MI355_DT_FP8_E4M3FN) return launch_t2<fp16_tag, fp8_tag, 256>(p, ws_prefix, skip_combine, s);
+    return "MFMA kernel: unsupported (q_dtype, kv_dtype) pair";
   }
   if (p.dim != 128) return "MFMA kernel: unsupported head dim";
   if (q_dtype == MI355_DT_BF16 && kv_dtype == MI355_DT_BF16) return launch_t2<bf16_tag, bf16_tag, 128>(p, ws_prefix, skip_combine, s);
