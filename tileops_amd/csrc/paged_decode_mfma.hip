@@ -899,7 +899,8 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   // loop phases and wall-clock start/end stamps, eight floats per wave written behind the workspace proper.
   uint64_t tm_issue = 0, tm_wait = 0, tm_comp = 0, tm_seg = 0, tm_mark = __builtin_readcyclecounter();
   const uint64_t tm_loop0 = tm_mark;
-#define TM(acc) { uint64_t now_ = __builtin_readcyclecounter(); acc += now_ - tm_mark; tm_mark = now_; }
+  // (the scheduling barriers keep the compiler from moving vector work of one phase across the stamp of the next)
+#define TM(acc) { __builtin_amdgcn_sched_barrier(0); uint64_t now_ = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); acc += now_ - tm_mark; tm_mark = now_; }
 #else
 #define TM(acc)
 #endif
