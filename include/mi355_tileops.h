@@ -30,7 +30,8 @@ extern "C" {
 /* kernel selection for mi355_gqa_paged_decode(): which implementation serves the call */
 #define MI355_KERNEL_AUTO 0    /* MFMA kernel when the shape qualifies, else the generic one */
 #define MI355_KERNEL_GENERIC 1 /* VALU kernel: any head_dim in {64,128,256}, any page size, any group */
-#define MI355_KERNEL_MFMA 2    /* MFMA kernel; MI355_EUNSUPPORTED if the shape does not qualify */
+#define MI355_KERNEL_MFMA 2    /* MFMA kernel (head_dim 64/128/256, 16-bit or FP8 cache, page size 16 or a multiple of 32);
+                                  MI355_EUNSUPPORTED if the shape does not qualify */
 /* Measurement aid, OR-ed into the selector: launch the attention kernel only and leave the partial results in
  * the workspace unmerged (the output is then incomplete).  Lets a benchmark time the dominant kernel alone. */
 #define MI355_KERNEL_FLAG_SKIP_COMBINE 0x100
