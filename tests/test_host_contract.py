@@ -322,6 +322,20 @@ def test_workspace_planning_is_host_only_and_reports_errors():
         native.decode_workspace(1, 1, 32, 8, 96, 64, 4, torch.bfloat16, torch.bfloat16)
     with pytest.raises(ValueError, match="must equal q_dtype"):
         native.decode_workspace(1, 1, 32, 8, 128, 64, 4, torch.bfloat16, torch.float16)
+    # the MFMA kernel cuts the tile stream so that every compute unit holds eight waves (four at head dim 256)
+    fp8 = torch.float8_e4m3fn
+    assert [native.decode_workspace(64, 1, 32, 8, d, 64, 128, torch.bfloat16, fp8, 0, native.KERNEL_MFMA)[1:] for d in (64, 128, 256)] == \
+        [(256, native.KERNEL_MFMA), (256, native.KERNEL_MFMA), (128, native.KERNEL_MFMA)]
+    # prefill: the fused-RoPE call adds room for the rotated queries, an FP8 cache two fp32 result sets to merge
+    plain = native.prefill_paged_workspace(8, 512, 4096, 32, 8, 128, 64, 72, torch.bfloat16, torch.bfloat16)
+    assert native.prefill_paged_rope_workspace(8, 512, 4096, 32, 8, 128, 64, 72, torch.bfloat16) == plain + 4096 * 32 * 128 * 2
+    assert native.prefill_paged_workspace(8, 512, 4096, 32, 8, 128, 64, 72, torch.bfloat16, fp8) >= plain + 2 * 4096 * 32 * 128 * 4
+    with pytest.raises(ValueError, match="heads must be divisible by heads_kv"):
+        native.prefill_paged_workspace(8, 512, 4096, 30, 8, 128, 64, 72, torch.bfloat16, torch.bfloat16)
+    with pytest.raises(ValueError, match="total_q must be non-negative"):
+        native.prefill_paged_rope_workspace(8, 512, -1, 32, 8, 128, 64, 72, torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="head dim 96"):
+        native.prefill_paged_workspace(8, 512, 4096, 32, 8, 96, 64, 72, torch.bfloat16, torch.bfloat16)
     lib = native.load()
     rc = lib.mi355_gqa_paged_decode(None, None, None, None, None, None, None, 1, None, None, 0, 1, 1, 32, 8, 128, 64, 64,
                                     native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, 0, 0, None)
