@@ -208,6 +208,32 @@ def test_fp8_cache_at_head_dims_64_and_256_on_the_mfma_kernel(dtype, page, q_len
     _run_and_compare(op, case, page, 3e-2, **({} if q_len == 1 else {"is_causal": True}))
 
 
+@pytest.mark.parametrize(
+    "heads, heads_kv, dim, fp8, lens",
+    [
+        pytest.param(8, 1, 128, True, [70001], id="one-kv-head-fp8-2048-partitions"),
+        pytest.param(32, 4, 128, False, [40000], id="256-partitions"),
+        pytest.param(32, 4, 128, False, [333, 0], id="fewer-tiles-than-partitions"),
+        pytest.param(16, 2, 64, False, [3000], id="head-dim-64-fewer-tiles-than-partitions"),
+        pytest.param(16, 2, 256, True, [9001, 5], id="head-dim-256-fp8-two-sequences"),
+        pytest.param(64, 8, 128, True, [33, 20000, 1], id="three-sequences-one-long"),
+    ],
+)
+def test_few_sequences_spread_over_hundreds_of_partitions(heads, heads_kv, dim, fp8, lens):
+    """Batch 1-3: every sequence spans far more than 64 partitions of the tile stream on average, which takes the
+    sixteen-wave merge (four LSEs per lane, lane groups on different partitions, the tail loop beyond 256 partitions,
+    and -- with fewer tiles than partitions -- the walk over the partitions that own a tile)."""
+    require_gfx950()
+    case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, torch.bfloat16, fp8=fp8, seed=71)
+    op = PagedOp(len(lens), heads, heads_kv, case[1].shape[0], dim, 64)
+    assert _serves(op, "gqa_decode_paged_mfma_kernel", torch.bfloat16, fp8)
+    _force(op, "gqa_decode_paged_mfma_kernel")
+    n_parts = native.decode_workspace(len(lens), 1, heads, heads_kv, dim, 64, case[4].shape[1], torch.bfloat16,
+                                      torch.float8_e4m3fn if fp8 else torch.bfloat16, 0, native.KERNEL_MFMA)[1]
+    assert n_parts > 64 * len(lens)
+    _run_and_compare(op, case, 64, 3e-2 if fp8 else 2e-2)
+
+
 def _serves(op, key, dtype, fp8):
     call = op.attention_call(dtype, torch.float8_e4m3fn if fp8 else None, torch.device(DEV, 0))
     return op.kernel_map[key].refusal(call) is None

@@ -1100,6 +1100,142 @@ __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __
   store(acc0 * inv, acc1 * inv, W > 0.f ? M + log2f(W) : -INFINITY);
 }
 
+// The same merge for calls whose sequences span very many partitions each (batch-1 long-context decode).
+// The waves of a workgroup work on one (sequence, kv head, query row) at a time.  A lane owns four consecutive head
+// elements, so 32 lanes (16 at head dim 64) cover a partial row and the two (four) lane groups of a wave take different
+// partitions with one 16-byte load each.  Every wave first fetches up to four LSEs per lane (the first 256 partitions,
+// one round trip), forms the maximum and the sum of weights, and meanwhile has its first eight row loads in flight;
+// the weighted sums of the groups meet through lane shuffles, those of the waves in LDS.  With 16 waves a sequence
+// spread over 256 partitions (batch-1 long-context decode) is merged in one round of loads.  When fewer tiles than
+// partitions exist, only the partitions that own a tile (one each) are visited.
+constexpr int kCombinePre = 8;   // row loads in flight per wave
+constexpr int kCombineLse = 4;   // LSEs kept per lane (first 64 * 4 partitions of the sequence)
+
+template <typename QT, int kCombineWaves>
+__device__ __forceinline__ void combine_row_wide(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x4 (*red)[64], int b, int row_all, int4 rec) {
+  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
+  const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
+  const int s = r / p.group, gi = r - s * p.group;
+  if (p.cu_q && r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
+  const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
+  const int hd = p.dim;
+  const int lpp = (hd < 128 ? hd : 128) >> 2;     // lanes per partial row (blockIdx.z picks the half of a 256-wide head)
+  const int ngrp = 64 / lpp, grp = lane / lpp;    // lane groups of a wave: each takes its own partition
+  const int dl = 4 * (lane - grp * lpp) + 128 * (int)blockIdx.z;
+  auto store = [&](f32x4 a, float lse) {
+    if (grp != 0) return;
+    if (p.final_o) {
+      *(f32x4*)(p.final_o + orow * hd + dl) = a;
+      if (lane == 0 && blockIdx.z == 0) p.final_lse[orow] = lse;
+    } else {
+      u32x2 w;
+      w[0] = Mma<QT>::pack(a[0], a[1]);
+      w[1] = Mma<QT>::pack(a[2], a[3]);
+      *(u32x2*)((uint16_t*)p.out + orow * hd + dl) = w;
+    }
+  };
+  const int p_first = rec.y, p_last = rec.z;
+  if (p_first < 0) {  // empty sequence: the attention kernel never visits it
+    if (wave == 0) store(f32x4{0.f, 0.f, 0.f, 0.f}, -INFINITY);
+    return;
+  }
+  const bool gaps = (rec.w & 2) != 0, first_in_slot1 = (rec.w & 1) != 0;  // (rec is wave-uniform: see the caller)
+  const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
+  // fewer tiles than partitions: the sequence's tiles sit one to a partition, the partitions in between own nothing;
+  // tile t then belongs to partition ((t + 1) * n_parts - 1) / T, and (t + 1) * n_parts stays far below 2^31
+  const uint32_t T = gaps ? (uint32_t)uni(((const int4*)ws_prefix)[p.batch].x) : 1u, NP = (uint32_t)p.n_parts;
+  const int n = gaps ? uni(((const int4*)ws_prefix)[b + 1].x) - rec.x : p_last - p_first + 1;
+  auto slot_at = [&](int i) {
+    const int ii = i < n ? i : n - 1;
+    int pp = p_first + ii;
+    if (gaps) pp = (int)(((uint32_t)(rec.x + ii + 1) * NP - 1u) / T);
+    return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all;
+  };
+  constexpr int PRE = kCombinePre, KL = kCombineLse;
+  // few partitions (the usual case when many sequences share the chip): one wave does it all
+  const int nw = n <= PRE * ngrp ? 1 : kCombineWaves;
+  if (wave >= nw) return;
+  // this wave's first row loads go out together with the LSEs, before any weight is known; load j of wave w covers
+  // partitions (j*nw + w)*ngrp .. +ngrp-1 of the sequence, one per lane group
+  f32x4 rows[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; i++) rows[i] = *(const f32x4*)(p.part_o + slot_at((i * nw + wave) * ngrp + grp) * hd + dl);
+  float lse[KL];
+#pragma unroll
+  for (int k = 0; k < KL; k++) lse[k] = 64 * k + lane < n ? p.part_lse[slot_at(64 * k + lane)] : -INFINITY;
+  float M = fmaxf(fmaxf(lse[0], lse[1]), fmaxf(lse[2], lse[3]));
+  static_assert(KL == 4, "four LSEs per lane");
+  for (int base = 64 * KL; base < n; base += 64) M = fmaxf(M, base + lane < n ? p.part_lse[slot_at(base + lane)] : -INFINITY);
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) M = fmaxf(M, __shfl_xor(M, m, 64));
+  float wk[KL], W = 0.f;
+#pragma unroll
+  for (int k = 0; k < KL; k++) {
+    wk[k] = (M != -INFINITY && lse[k] != -INFINITY) ? fast_exp2(lse[k] - M) : 0.f;  // weight of partition 64k + lane
+    W += wk[k];
+  }
+  if (M != -INFINITY)
+    for (int base = 64 * KL; base < n; base += 64) W += base + lane < n ? fast_exp2(p.part_lse[slot_at(base + lane)] - M) : 0.f;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) W += __shfl_xor(W, m, 64);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (W > 0.f) {
+    for (int j0 = 0; (j0 * nw + wave) * ngrp < n; j0 += PRE) {
+      float wt[PRE];
+#pragma unroll
+      for (int i = 0; i < PRE; i++) {
+        const int base = ((j0 + i) * nw + wave) * ngrp, idx = base + grp;  // base is wave-uniform and a multiple of ngrp
+        if (base < 64 * KL) {
+          const int k = base >> 6;
+          const float src = k == 0 ? wk[0] : (k == 1 ? wk[1] : (k == 2 ? wk[2] : wk[3]));
+          wt[i] = __shfl(src, idx & 63, 64);  // (0 for indices past the last partition)
+        } else {
+          wt[i] = idx < n ? fast_exp2(p.part_lse[slot_at(idx)] - M) : 0.f;
+        }
+        if (j0 > 0) rows[i] = *(const f32x4*)(p.part_o + slot_at(idx) * hd + dl);
+      }
+#pragma unroll
+      for (int i = 0; i < PRE; i++)
+        if (wt[i] != 0.f) acc += wt[i] * rows[i];  // an unwritten slot may hold anything, NaN included
+    }
+  }
+  // the lane groups of the wave, then the waves
+  if (ngrp == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], 16, 64);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) acc[e] += __shfl_xor(acc[e], 32, 64);
+  if (nw > 1) {  // uniform over the workgroup: either every wave is here or only wave 0 exists
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int w = 1; w < kCombineWaves; w++) acc += red[w][lane];
+  }
+  const float inv = W > 0.f ? 1.0f / W : 0.f;
+  store(acc * inv, W > 0.f ? M + log2f(W) : -INFINITY);
+}
+
+// grid (ceil(heads_kv*rows / rows_per_wg), batch, halves of a 256-wide head): a workgroup takes rows_per_wg consecutive
+// rows of one sequence.  With thousands of rows per sequence (prefill chunks) most sequences lie inside one partition
+// and need no merge at all: the workgroup reads the sequence's record once and leaves, instead of one workgroup per row
+// doing so (131 072 of them took 28 us on an 8 x 512-row call).
+template <typename QT, int kCombineWaves>
+__global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_wide_kernel(const DecodeParams p, const int* __restrict__ ws_prefix,
+                                                                                       int rows_per_wg) {
+  __shared__ f32x4 red[kCombineWaves][64];
+  const int b = blockIdx.y;
+  const int4 recv = ((const int4*)ws_prefix)[b];  // the only load everything else depends on
+  const int4 rec = {uni(recv.x), uni(recv.y), uni(recv.z), uni(recv.w)};  // scalar: every branch on it is a scalar branch
+  if (rec.y >= 0 && rec.y == rec.z) return;  // one wave covered the whole sequence and wrote the output itself
+  const int row_end = min((int)(blockIdx.x + 1) * rows_per_wg, p.heads_kv * p.rows);
+  for (int row_all = blockIdx.x * rows_per_wg; row_all < row_end; row_all++) {
+    combine_row_wide<QT, kCombineWaves>(p, ws_prefix, red, b, row_all, rec);
+    if (kCombineWaves > 1 && row_all + 1 < row_end) __syncthreads();  // red[] is reused by the next row
+  }
+}
+
 // Unshared waves per workgroup: with a 16-bit cache a stage is 16 KiB, two stages x four waves fill the LDS of a CU.  With an
 // fp8 cache a stage is half that, so eight waves fit: the eight kv heads of a page set then sit in one CU and the
 // 32-byte sectors of the scale rows (all heads of a token) are fetched once instead of once per workgroup.
@@ -1127,14 +1263,17 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hipGetErrorString(e);
   if (skip_combine) return nullptr;
-  // four waves per row when sequences span many partitions on average, one otherwise (fewer waves to launch)
+  // one wave per row as a rule, four when sequences span more than eight partitions on average; beyond 64 the wide
+  // kernel (sixteen waves, 16-byte lanes, one round of loads), which costs more per row and pays only there
   // rows per workgroup: one while the call has few rows (decode), more once a workgroup per row would mean tens of
   // thousands of workgroups (prefill chunks)
   const int rows_all = p.heads_kv * p.rows;
   int rows_per_wg = 1;
   while ((int64_t)rows_all * p.batch / rows_per_wg > 8192 && rows_per_wg < 64) rows_per_wg *= 2;
   const dim3 cgrid((rows_all + rows_per_wg - 1) / rows_per_wg, p.batch, D > 128 ? 2 : 1);
-  if ((int64_t)p.n_parts > 8 * (int64_t)p.batch)
+  if ((int64_t)p.n_parts > 64 * (int64_t)p.batch)
+    hipLaunchKernelGGL((paged_decode_mfma_combine_wide_kernel<QT, 16>), cgrid, dim3(1024), 0, s, p, ws_prefix, rows_per_wg);
+  else if ((int64_t)p.n_parts > 8 * (int64_t)p.batch)
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
   else
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), cgrid, dim3(64), 0, s, p, ws_prefix, rows_per_wg);
