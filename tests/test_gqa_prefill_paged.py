@@ -274,6 +274,32 @@ def test_head_dim_128_empty_chunks_empty_caches_and_both_kernels(kernel, fp8, dt
 
 
 @pytest.mark.gpu
+def test_validate_inputs_false_skips_the_device_reads_and_nothing_else():
+    """Same result bit for bit; a call whose cu_seqlens_q is inconsistent is then no longer caught on the host (the
+    check needs a device read), while shape and dtype mistakes still are."""
+    require_gfx950()
+    case = _case([33, 48], [67, 80], 8, 2, 64, torch.float16)
+    kw = dict(batch=2, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64)
+    dev = [t.to(DEV) for t in case]
+    out_checked = PrefillOp(**kw)(*[t.clone() for t in dev], 48)
+    fast = PrefillOp(**kw, validate_inputs=False)
+    torch.cuda.synchronize()
+    syncs_before = torch.cuda.get_sync_debug_mode()
+    torch.cuda.set_sync_debug_mode("error")  # any host read of device memory raises
+    try:
+        out_fast = fast(*[t.clone() for t in dev], 48)
+    finally:
+        torch.cuda.set_sync_debug_mode(syncs_before)
+    assert torch.equal(out_checked, out_fast)
+    with pytest.raises(ValueError, match="block_table shape"):
+        fast(*dev[:9], dev[9][:, :4].contiguous(), 48)
+    bad_cu = dev[7].clone()
+    bad_cu[0] = 1
+    with pytest.raises(ValueError, match=r"cu_seqlens_q\[0\] must be 0"):
+        PrefillOp(**kw)(*dev[:7], bad_cu, *dev[8:], 48)
+
+
+@pytest.mark.gpu
 def test_prefill_rejects_bad_calls():
     require_gfx950()
     case = [t.to(DEV) for t in _case([4, 4], [10, 10], 8, 2, 64, torch.float16)]
