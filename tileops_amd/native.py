@@ -153,12 +153,24 @@ def dtype_code(dtype: torch.dtype) -> int:
     raise ValueError(f"dtype {dtype} has no MI355X kernel (bfloat16, float16, float8_e4m3fn)")
 
 
+_GFX950_BY_INDEX: dict[int, bool] = {}  # a device's architecture does not change: asked once per device index
+
+
 def is_gfx950(device: torch.device) -> bool:
     """True iff *device* is a ROCm GPU whose architecture is gfx950 (MI350X / MI355X)."""
-    if device.type != "cuda" or torch.version.hip is None or not torch.cuda.is_available():
+    if device.type != "cuda" or torch.version.hip is None:
+        return False
+    index = device.index
+    known = _GFX950_BY_INDEX.get(index) if index is not None else None
+    if known is not None:
+        return known
+    if not torch.cuda.is_available():
         return False
     name = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
-    return name.split(":")[0] == "gfx950"
+    answer = name.split(":")[0] == "gfx950"
+    if index is not None:
+        _GFX950_BY_INDEX[index] = answer
+    return answer
 
 
 def require_gfx950(device: torch.device) -> None:

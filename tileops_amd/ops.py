@@ -120,8 +120,15 @@ class _PagedDecodeOp(Op):
             # an external target serves this instance: its builder chooses among its own kernels
             return self.get_or_build_kernel("gqa_decode_paged_kernel", inputs)
         device = next((t.device for t in inputs if t is not None), None)
-        call = self.attention_call(dtype, kv_dtype, device)
-        key = self.select_kernel_key(PAGED_DECODE_KEYS, call)
+        # selection is a function of the call and of the kernel map: settled once per (dtypes, device, map), like the
+        # reference's once-per-dtype kernel choice (ops/attention/gqa.py:1389-1408)
+        memo_key = (dtype, kv_dtype, device, tuple(self.kernel_map.items()))
+        memo = self.__dict__.setdefault("_selected_keys", {})
+        hit = memo.get(memo_key)
+        if hit is None:
+            call = self.attention_call(dtype, kv_dtype, device)
+            hit = memo[memo_key] = (self.select_kernel_key(PAGED_DECODE_KEYS, call), call)
+        key, call = hit
 
         def build():
             return self.kernel_map[key](
