@@ -980,29 +980,39 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
 // trips instead of one per partition.  64*kCombineWaves threads; the launcher takes the one-wave instance when the
 // average sequence spans at most eight partitions.
 template <typename QT, int kCombineWaves>
-__device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec);
+__device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec,
+                                            int wave);
 
 // grid (ceil(heads_kv*rows / rows_per_wg), batch, halves of a 256-wide head): a workgroup takes rows_per_wg consecutive
 // rows of one sequence.  With thousands of rows per sequence (prefill chunks) most sequences lie inside one partition
 // and need no merge at all: the workgroup reads the sequence's record once and leaves, instead of one workgroup per row
 // doing so (131 072 of them took 28 us on an 8 x 512-row call).
 template <typename QT, int kCombineWaves>
-__global__ __launch_bounds__(64 * kCombineWaves) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix,
-                                                                                       int rows_per_wg) {
+__global__ __launch_bounds__(256) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix, int rows_per_wg) {
+  // always four waves: either they share one row at a time (kCombineWaves == 4) or each takes every fourth row of the
+  // workgroup's range on its own (kCombineWaves == 1)
+  static_assert(kCombineWaves == 1 || kCombineWaves == 4, "one or four waves per row");
   __shared__ f32x2 red[kCombineWaves][64];
   const int b = blockIdx.y;
   const int4 rec = ((const int4*)ws_prefix)[b];  // the only load everything else depends on
   if (rec.y >= 0 && rec.y == rec.z) return;  // one wave covered the whole sequence and wrote the output itself
   const int row_end = min((int)(blockIdx.x + 1) * rows_per_wg, p.heads_kv * p.rows);
-  for (int row_all = blockIdx.x * rows_per_wg; row_all < row_end; row_all++) {
-    combine_row<QT, kCombineWaves>(p, ws_prefix, red, b, row_all, rec);
-    if (kCombineWaves > 1 && row_all + 1 < row_end) __syncthreads();  // red[] is reused by the next row
+  const int phys_wave = uni(threadIdx.x >> 6);
+  if constexpr (kCombineWaves == 1) {
+    for (int row_all = blockIdx.x * rows_per_wg + phys_wave; row_all < row_end; row_all += 4)
+      combine_row<QT, 1>(p, ws_prefix, red, b, row_all, rec, 0);
+  } else {
+    for (int row_all = blockIdx.x * rows_per_wg; row_all < row_end; row_all++) {
+      combine_row<QT, kCombineWaves>(p, ws_prefix, red, b, row_all, rec, phys_wave);
+      if (row_all + 1 < row_end) __syncthreads();  // red[] is reused by the next row
+    }
   }
 }
 
 template <typename QT, int kCombineWaves>
-__device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec) {
-  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
+__device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec,
+                                            int wave) {  // wave = this wave's index among the kCombineWaves that share the row
+  const int lane = threadIdx.x & 63;
   const int kvh = row_all / p.rows, r = row_all - kvh * p.rows;
   const int s = r / p.group, gi = r - s * p.group;
   if (p.cu_q && r >= q_len_of(p, b) * p.group) return;  // packed queries: this sequence has fewer rows
@@ -1265,18 +1275,19 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   if (skip_combine) return nullptr;
   // one wave per row as a rule, four when sequences span more than eight partitions on average; beyond 64 the wide
   // kernel (sixteen waves, 16-byte lanes, one round of loads), which costs more per row and pays only there
-  // rows per workgroup: one while the call has few rows (decode), more once a workgroup per row would mean tens of
-  // thousands of workgroups (prefill chunks)
+  // rows per workgroup: one per wave while the call has few rows (decode), more once that would mean tens of thousands
+  // of workgroups (prefill chunks)
   const int rows_all = p.heads_kv * p.rows;
-  int rows_per_wg = 1;
+  const bool wide = (int64_t)p.n_parts > 64 * (int64_t)p.batch, four = !wide && (int64_t)p.n_parts > 8 * (int64_t)p.batch;
+  int rows_per_wg = (wide || four) ? 1 : 4;
   while ((int64_t)rows_all * p.batch / rows_per_wg > 8192 && rows_per_wg < 64) rows_per_wg *= 2;
   const dim3 cgrid((rows_all + rows_per_wg - 1) / rows_per_wg, p.batch, D > 128 ? 2 : 1);
-  if ((int64_t)p.n_parts > 64 * (int64_t)p.batch)
+  if (wide)
     hipLaunchKernelGGL((paged_decode_mfma_combine_wide_kernel<QT, 16>), cgrid, dim3(1024), 0, s, p, ws_prefix, rows_per_wg);
-  else if ((int64_t)p.n_parts > 8 * (int64_t)p.batch)
+  else if (four)
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
   else
-    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), cgrid, dim3(64), 0, s, p, ws_prefix, rows_per_wg);
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
   e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
