@@ -97,6 +97,8 @@ struct Extras {
   int scale_per_tensor = 0;
   float* final_o = nullptr;
   float* final_lse = nullptr;
+  const float* init_o = nullptr;
+  const float* init_lse = nullptr;
 };
 
 // One decode call, paged (block_table/seqlens given) or contiguous (contig_stride > 0, uniform_len).
@@ -142,6 +144,8 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
   p.scale_per_tensor = ex.scale_per_tensor;
   p.final_o = ex.final_o;
   p.final_lse = ex.final_lse;
+  p.init_o = ex.init_o;
+  p.init_lse = ex.init_lse;
   p.out = out;
   p.part_o = (float*)workspace;
   p.part_lse = (float*)((char*)workspace + plan.part_o_bytes);
@@ -349,13 +353,25 @@ int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new,
   eb.cu_q = cu_seqlens_q;
   eb.len_excludes_new = 1;  // with no seqlens array: length = the chunk's own length
   eb.kv_starts = cu_seqlens_q;
-  eb.final_o = o_b;
-  eb.final_lse = lse_b;
+  // When the second pass runs on the MFMA kernel it starts every row from the first pass's result and writes the
+  // output itself; otherwise it leaves a second fp32 result and merge_two_kernel joins the two.
+  Plan plan_a, plan_b;
+  rc = prefill_plans(batch, max_seqlen_q, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, cache_dtype, kernel, &plan_a, &plan_b);
+  if (rc) return rc;
+  const bool carried = plan_b.kernel == MI355_KERNEL_MFMA;
+  if (carried) {
+    eb.init_o = o_a;
+    eb.init_lse = lse_a;
+  } else {
+    eb.final_o = o_b;
+    eb.final_lse = lse_b;
+  }
   rc = run_decode(q, k_new, v_new, nullptr, nullptr, nullptr, nullptr, ((int64_t)max_seqlen_q + kContigTile - 1) / kContigTile, 0, 0,
                   out, workspace, need - 2 * fin, batch, max_seqlen_q, heads, heads_kv, dim, kContigTile,
                   ((total_q + kContigTile - 1) / kContigTile) * kContigTile, q_dtype, q_dtype, sm_scale, softcap, causal, 0, kernel,
                   hip_stream, eb);
   if (rc) return rc;
+  if (carried) return MI355_OK;
   err = launch_merge_two(o_a, lse_a, o_b, lse_b, out, total_q * heads, dim, q_dtype, s);
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
   return MI355_OK;

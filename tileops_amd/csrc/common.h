@@ -37,6 +37,11 @@ struct DecodeParams {
   // instead of 16-bit rows in out, so that two calls over disjoint key sets can be merged afterwards.
   float* final_o;
   float* final_lse;
+  // MFMA kernel: when set, every query row starts from this earlier result over a disjoint key set (fp32 rows and
+  // log2-domain log-sum-exp as written through final_o / final_lse) instead of from nothing, so the call's output is
+  // already the merge of both.
+  const float* init_o;
+  const float* init_lse;
   void* out;
   float* part_o;    // workspace: normalised partial outputs, fp32
   float* part_lse;  // workspace: log2-domain log-sum-exp per partial (-inf = empty)

@@ -631,6 +631,31 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
 #pragma unroll
       for (int db = 0; db < NDB; db++) o_acc[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    if (p.init_o && cu.j == 0) {
+      // Carried state: the segment opens the sequence, so its rows take over the earlier result.  A normalised row O
+      // with log-sum-exp L is the state (reference m = L, sum l = 1, accumulator O); the sum is kept in the g == 0
+      // lanes because the final sum adds the four lane groups.  L = -inf (no earlier keys) leaves the empty state.
+#pragma unroll
+      for (int rb = 0; rb < NRB; rb++) {
+        int r = rg * (16 * NRB) + rb * 16 + c;
+        bool valid = r < seg_q_len * p.group;
+        int s = valid ? r / p.group : 0, gi = valid ? r - s * p.group : 0;
+        const int64_t orow = (seg_q_row0 + s) * p.heads + kvh * p.group + gi;
+        const float l0 = valid ? p.init_lse[orow] : -INFINITY;
+        if (l0 != -INFINITY) {
+          m_run[rb] = l0;
+          l_run[rb] = g == 0 ? 1.f : 0.f;
+#pragma unroll
+          for (int db = 0; db < NDB; db++) o_acc[rb][db] = *(const f32x4*)(p.init_o + orow * D + 16 * db + 4 * g);
+        }
+      }
+#pragma unroll
+      for (int rb = 0; rb < NRB; rb++) {
+        asm volatile("" : "+v"(m_run[rb]));
+#pragma unroll
+        for (int db = 0; db < NDB; db++) asm volatile("" : "+v"(o_acc[rb][db]));  // land here, not in the loop
+      }
+    }
     {
       int lm = limit[0];
 #pragma unroll
