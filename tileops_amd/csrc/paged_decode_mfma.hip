@@ -570,7 +570,6 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   const uint32_t q_sign = p.negate_q ? (QK8 ? 0x80808080u : 0x80008000u) : 0u;
   float q_scale[NRB];  // QK8: the power of two taken out of the lane's query row (row c of each row block)
 
-  int seg_limit_max = 0;     // first token that none of this wave's rows sees (wave-uniform): tiles from there on are skipped
   int seg_q_len = p.q_len;   // query tokens of the sequence being processed (varies with packed queries)
   int64_t seg_q_row0 = 0;    // its first row in q / out
   auto begin_segment = [&](const Cursor& cu) __attribute__((always_inline)) {
@@ -655,14 +654,6 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
 #pragma unroll
         for (int db = 0; db < NDB; db++) asm volatile("" : "+v"(o_acc[rb][db]));  // land here, not in the loop
       }
-    }
-    {
-      int lm = limit[0];
-#pragma unroll
-      for (int rb = 1; rb < NRB; rb++) lm = max(lm, limit[rb]);
-#pragma unroll
-      for (int m = 1; m < 64; m <<= 1) lm = max(lm, __shfl_xor(lm, m, 64));
-      seg_limit_max = uni(lm);
     }
     // Make the query loads land here: an empty asm that "modifies" each register forces the compiler to put
     // its own vmcnt wait in this (rare) block instead of in the steady-state loop, where such a wait would
@@ -961,21 +952,15 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         TM(tm_wait)
         if (LATE) issue_ahead(ring);
         TM(tm_issue)
-        if (__builtin_expect(cc.j * kCT >= seg_limit_max, 0)) {
-          // Causal chunk: the tile lies behind the last key any row of this wave sees (or the wave is an idle row
-          // group of its ring).  It took part in the fetch and the barrier; there is nothing to add.
+        moved = run_score_step(ring);
+        if constexpr ((SH && D <= 128) || (FP8 && NRB == 2)) {
+          // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
+          if (__builtin_expect(moved, 0)) rescale();
           moved = false;
         } else {
-          moved = run_score_step(ring);
-          if constexpr ((SH && D <= 128) || (FP8 && NRB == 2)) {
-            // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
-            if (__builtin_expect(moved, 0)) rescale();
-            moved = false;
-          } else {
-            if (__builtin_expect(moved, 0)) break;
-          }
-          value_step();
+          if (__builtin_expect(moved, 0)) break;
         }
+        value_step();
         TM(tm_comp)
         ++u;
         ++cc.j;
