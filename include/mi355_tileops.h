@@ -32,9 +32,6 @@ extern "C" {
 #define MI355_KERNEL_GENERIC 1 /* VALU kernel: any head_dim in {64,128,256}, any page size, any group */
 #define MI355_KERNEL_MFMA 2    /* MFMA kernel (head_dim 64/128/256, 16-bit or FP8 cache, page size 16 or a multiple of 32);
                                   MI355_EUNSUPPORTED if the shape does not qualify */
-/* Measurement aid, OR-ed into the selector: launch the attention kernel only and leave the partial results in
- * the workspace unmerged (the output is then incomplete).  Lets a benchmark time the dominant kernel alone. */
-#define MI355_KERNEL_FLAG_SKIP_COMBINE 0x100
 
 /* error codes */
 #define MI355_OK 0
@@ -42,7 +39,8 @@ extern "C" {
 #define MI355_EUNSUPPORTED (-2) /* legal call, but no kernel in this library serves it */
 #define MI355_EWORKSPACE (-3)   /* workspace pointer missing or too small */
 #define MI355_ELAUNCH (-4)      /* HIP reported an error at launch */
-#define MI355_EDEVICE (-5)      /* current device is not gfx950 */
+#define MI355_EDEVICE (-5)      /* no current HIP device, or it is not gfx950: returned by every entry point that would
+                                   launch, before anything is launched (workspace queries touch no device) */
 
 /* Version of this ABI (MI355_ABI_VERSION of the library that was loaded). */
 int mi355_abi_version(void);
@@ -96,6 +94,8 @@ int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_
  *   num_split    as num_split_in above;  kernel as above
  *
  * Sequences with seqlens[b] == 0 produce zeros.  Tokens not addressed by (block_table, seqlens) are never read.
+ * Lengths are clamped on the device to [0, bt_row_stride * page_size], what one block-table row can address, so a
+ * corrupt seqlens[b] cannot make a kernel read the table past the sequence's row; page ids are clamped into the pool.
  */
 int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const float* k_scale,
                            const float* v_scale, const int32_t* seqlens, const int32_t* block_table,
@@ -134,8 +134,8 @@ int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k
  * Packed GQA prefill chunk with paged KV-cache append: one call = one forward of
  * GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp (src/tileops/ops/attention/gqa.py:1072-1140 ->
  * GQAPrefillPagedWithKVCacheFwdKernel / GQAPrefillPagedWithFP8KVCacheFwdKernel,
- * src/tileops/kernels/attention/gqa_fwd.py:600-1000 and :1005-1460).  Fused RoPE (the third reference kernel) is
- * not served.
+ * src/tileops/kernels/attention/gqa_fwd.py:600-1000 and :1005-1460).  The third reference kernel, fused RoPE, is
+ * mi355_gqa_prefill_paged_rope() below.
  *
  *   q              [total_q, heads, dim] q_dtype: the chunks of all sequences packed; sequence b owns rows
  *                  [cu_seqlens_q[b], cu_seqlens_q[b+1])
@@ -153,7 +153,8 @@ int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k
  *   causal         query i of a chunk sees the old tokens and chunk tokens j <= i (gqa_fwd.py:1247-1256); 0: all of them
  * Attention runs over the dequantised old tokens and the *unquantised* chunk (as the reference: :1180-1245): with an fp8
  * cache that is two passes (pages, then k_new/v_new) whose fp32 results are merged by log-sum-exp.
- * Sequences with an empty chunk produce no output rows and append nothing.
+ * Sequences with an empty chunk produce no output rows and append nothing.  A chunk token whose position
+ * cache_seqlens[b] + i the block-table row cannot address (negative, or page index >= bt_row_stride) is not appended.
  */
 int mi355_gqa_prefill_paged_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
                                       int page_size, int64_t max_pages_per_req, int q_dtype, int cache_dtype, int kernel,

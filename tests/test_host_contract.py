@@ -341,3 +341,38 @@ def test_workspace_planning_is_host_only_and_reports_errors():
                                     native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, 0, 0, None)
     assert rc == -1 and b"non-null" in lib.mi355_last_error()
     assert tileops_amd.__version__
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="needs a host without a GPU: the pointers below are made up")
+def test_entry_points_refuse_without_a_gfx950_device_before_launching():
+    """A call whose arguments pass validation still launches nothing when no gfx950 device is current: every launching
+    entry point returns MI355_EDEVICE with a message (the reference refuses by architecture before it builds a kernel,
+    src/tileops/kernels/kernel_base.py:98-112).  Argument errors keep precedence, workspace queries touch no device."""
+    lib = native.load()
+    header = (ROOT / "include" / "mi355_tileops.h").read_text()
+    edevice = int(re.search(r"#define MI355_EDEVICE \((-?\d+)\)", header).group(1))
+    fake = 0x10000  # aligned, never dereferenced
+    ws_bytes, n_parts, _ = native.decode_workspace(2, 1, 32, 8, 128, 64, 4, torch.bfloat16, torch.bfloat16, 0, native.KERNEL_MFMA)
+    rc = lib.mi355_gqa_paged_decode(fake, fake, fake, None, None, fake, fake, 4, fake, fake, ws_bytes, 2, 1, 32, 8, 128, 64, 64 * 8,
+                                    native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, 0, native.KERNEL_MFMA, None)
+    assert rc == edevice and b"gfx950" in lib.mi355_last_error()
+    rc = lib.mi355_gqa_decode(fake, fake, fake, None, None, fake, fake, 1 << 30, 2, 1, 32, 8, 128, 4096, 1000,
+                              native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, 0, native.KERNEL_GENERIC, None)
+    assert rc == edevice
+    rc = lib.mi355_gather_probe(fake, fake, fake, 4, fake, 2, 256, 2048, 64, 64 * 8, None)
+    assert rc == edevice
+    rc = lib.mi355_kv_append_fp8(fake, fake, fake, fake, fake, 4, 2, 8, 128, 64, 64 * 8, native.DT_BF16, None)
+    assert rc == edevice
+    need = native.prefill_paged_workspace(2, 16, 32, 32, 8, 128, 64, 4, torch.bfloat16, torch.bfloat16)
+    rc = lib.mi355_gqa_prefill_paged(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, 4, fake, fake, need, 2, 16, 32, 32, 8,
+                                     128, 64, 64 * 8, native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, native.KERNEL_AUTO, None)
+    assert rc == edevice
+    # an argument error is still reported first
+    rc = lib.mi355_gqa_paged_decode(fake, fake, fake, None, None, fake, fake, 4, fake, fake, ws_bytes, 2, 1, 30, 8, 128, 64, 64 * 8,
+                                    native.DT_BF16, native.DT_BF16, 1.0, 0.0, 1, 0, native.KERNEL_MFMA, None)
+    assert rc == -1
+    # the Python binding turns the code into the package's library error
+    q = torch.zeros(2, 32, 128, dtype=torch.bfloat16)
+    with pytest.raises(native.NativeLibraryError):
+        native._check(lib.mi355_gather_probe(fake, fake, fake, 4, fake, 2, 256, 2048, 64, 64 * 8, None))
+    assert "gfx950" in native.last_error() and q.device.type == "cpu"

@@ -1,8 +1,11 @@
 // extern "C" entry points of libmi355_tileops: argument validation, kernel choice, launch.
 // Never throws, never aborts, never synchronises, never allocates device memory.
+#include <limits.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+
+#include <atomic>
 
 #include "common.h"
 
@@ -18,6 +21,34 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
+}
+
+// Architecture of the current device, asked once per device: 1 = gfx950, -1 = something else, 0 = not asked yet.
+// The kernels are gfx950 code objects (direct-to-LDS loads, transpose reads, the 128-deep fp8 matrix instruction);
+// the reference refuses by architecture before building a kernel (src/tileops/kernels/kernel_base.py:98-112).
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_arch_ok[kMaxDevices];
+std::atomic<int> g_cu_count[kMaxDevices];
+
+int check_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+    (void)hipGetLastError();
+    return fail(MI355_EDEVICE, "no HIP device is current (these kernels need a gfx950 GPU)");
+  }
+  int known = dev < kMaxDevices ? g_arch_ok[dev].load(std::memory_order_relaxed) : 0;
+  if (known == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(MI355_EDEVICE, "cannot read the properties of HIP device %d", dev);
+    }
+    known = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    if (dev < kMaxDevices) g_arch_ok[dev].store(known, std::memory_order_relaxed);
+    if (known < 0) return fail(MI355_EDEVICE, "HIP device %d is %s; this library holds gfx950 (MI355X) code only", dev, prop.gcnArchName);
+  }
+  if (known < 0) return fail(MI355_EDEVICE, "HIP device %d is not a gfx950 (MI355X) GPU", dev);
+  return MI355_OK;
 }
 
 bool is_q_dtype(int d) { return d == MI355_DT_BF16 || d == MI355_DT_FP16; }
@@ -107,8 +138,8 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
                int uniform_len, void* out, void* workspace, size_t workspace_bytes, int batch, int q_len, int heads,
                int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale,
                float softcap, int causal, int num_split, int kernel, void* hip_stream, const Extras& ex = Extras()) {
-  const bool skip_combine = (kernel & MI355_KERNEL_FLAG_SKIP_COMBINE) != 0;
-  kernel &= ~MI355_KERNEL_FLAG_SKIP_COMBINE;
+  const bool skip_combine = (kernel & kKernelFlagSkipCombine) != 0;
+  kernel &= ~kKernelFlagSkipCombine;
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
   if (fp8 && (!k_scale || !v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale are required with an fp8 KV cache");
   if (!fp8 && (k_scale || v_scale)) return fail(MI355_EINVAL, "k_scale and v_scale must be null unless kv_dtype is fp8_e4m3fn");
@@ -125,6 +156,9 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
     if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
     if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
   }
+
+  rc = check_device();
+  if (rc) return rc;
 
   DecodeParams p;
   memset(&p, 0, sizeof(p));
@@ -158,6 +192,11 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
   p.group = heads / heads_kv;
   p.rows = q_len * p.group;
   p.n_pages = n_phys_tokens / page_size;
+  {
+    // what one block-table row (contiguous cache: one sequence's share, passed as bt_row_stride tiles) can address
+    const int64_t cap = bt_row_stride * (int64_t)page_size;
+    p.max_len = cap > INT_MAX ? INT_MAX : (int)cap;
+  }
   p.softcap = softcap;
   if (softcap > 0.f) {
     p.score_scale = sm_scale;
@@ -185,6 +224,25 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
 
 }  // namespace
 
+namespace mi355 {
+int device_cu_count() {
+  constexpr int kDefault = 256;  // MI355X: 8 XCDs x 32 compute units
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+    (void)hipGetLastError();
+    return kDefault;
+  }
+  int n = dev < kMaxDevices ? g_cu_count[dev].load(std::memory_order_relaxed) : 0;
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return kDefault;
+  }
+  if (dev < kMaxDevices) g_cu_count[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+}  // namespace mi355
+
 extern "C" {
 
 int mi355_abi_version(void) { return MI355_ABI_VERSION; }
@@ -199,7 +257,7 @@ int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_
   Plan plan;
   // softcap does not change the plan; the MFMA kernel serves both settings
   rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, max_blocks_per_seq, q_dtype, kv_dtype, 0.f, num_split_in,
-                 kernel & ~MI355_KERNEL_FLAG_SKIP_COMBINE, &plan);
+                 kernel & ~kKernelFlagSkipCombine, &plan);
   if (rc) return rc;
   if (workspace_bytes) *workspace_bytes = plan.part_o_bytes + plan.part_lse_bytes;
   if (num_split_out) *num_split_out = plan.kernel == MI355_KERNEL_GENERIC ? plan.max_splits : plan.n_parts;
@@ -319,6 +377,8 @@ int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new,
     if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
     if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
   }
+  rc = check_device();
+  if (rc) return rc;
   hipStream_t s = (hipStream_t)hip_stream;
   const char* err = launch_kv_append_chunk(k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens,
                                            block_table, bt_row_stride, batch, total_q, heads_kv, dim, page_size,
@@ -422,6 +482,8 @@ int mi355_gqa_prefill_paged_rope(const void* q, const void* k_new, const void* v
   if (!workspace) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got null", need);
   if (workspace_bytes < need) return fail(MI355_EWORKSPACE, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(MI355_EWORKSPACE, "workspace must be 256-byte aligned");
+  rc = check_device();
+  if (rc) return rc;
   void* q_rot = (char*)workspace + align256(base);
   const char* err = launch_rope_append_chunk(q, k_new, v_new, q_rot, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q,
                                              cache_seqlens, block_table, bt_row_stride, batch, total_q, heads, heads_kv, dim,
@@ -449,6 +511,7 @@ int mi355_gather_probe(const void* cache, const int32_t* seqlens, const int32_t*
   if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
   if (batch == 0 || max_len == 0) return MI355_OK;
   if (!cache || !seqlens || !block_table || !dense_out) return fail(MI355_EINVAL, "null pointer argument");
+  if (int rc = check_device()) return rc;
   const char* err = launch_gather_probe(cache, seqlens, block_table, bt_row_stride, dense_out, batch, max_len, row_bytes,
                                         page_size, n_phys_tokens / page_size, (hipStream_t)hip_stream);
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
@@ -468,6 +531,7 @@ int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int3
   if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
   if (batch == 0) return MI355_OK;
   if (!x_new || !cache || !scale || !seqlens || !block_table) return fail(MI355_EINVAL, "null pointer argument");
+  if (int rc = check_device()) return rc;
   const char* err = launch_kv_append_fp8(x_new, cache, scale, seqlens, block_table, bt_row_stride, batch, heads_kv, dim,
                                          page_size, n_phys_tokens / page_size, x_dtype, (hipStream_t)hip_stream);
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);

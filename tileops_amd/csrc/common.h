@@ -7,6 +7,11 @@
 
 namespace mi355 {
 
+// Measurement aid, OR-ed into the kernel selector of the decode entry points by this package's own benchmark: launch the
+// attention kernel only and leave the partial results in the workspace unmerged (the output is then incomplete), so
+// that the dominant kernel can be timed alone.  Not part of the public interface.
+constexpr int kKernelFlagSkipCombine = 0x100;
+
 constexpr float kLog2e = 1.4426950408889634f;
 // Finite stand-in for "-infinity" as the running maximum: exp2(-inf - kNegFloor) == 0 and
 // exp2(kNegFloor - kNegFloor) == 1, so empty tiles and empty splits never produce NaN.
@@ -49,6 +54,7 @@ struct DecodeParams {
   int group;        // heads / heads_kv
   int rows;         // q_len * group : query rows that share one kv head
   int64_t n_pages;  // n_phys_tokens / page_size
+  int max_len;      // tokens one block-table row (or one sequence's slot of a contiguous cache) can address: lengths are clamped to it
   float score_scale;  // sm_scale (softcap on) or sm_scale * log2e (softcap off)
   float softcap;      // 0 = off
   float cap_log2e;    // softcap * log2e
@@ -62,7 +68,9 @@ struct DecodeParams {
   int n_parts;
 };
 
-// Context length of sequence b: per-sequence array (paged cache) or one value for all (contiguous cache).
+// Context length of sequence b: per-sequence array (paged cache) or one value for all (contiguous cache), clamped to
+// [0, max_len] so that a corrupt length can neither run the kernels past the sequence's block-table row nor make the
+// tile-stream sums negative.
 __device__ __forceinline__ int q_len_of(const DecodeParams& p, int b) { return p.cu_q ? p.cu_q[b + 1] - p.cu_q[b] : p.q_len; }
 __device__ __forceinline__ int64_t q_row0_of(const DecodeParams& p, int b) { return p.cu_q ? (int64_t)p.cu_q[b] : (int64_t)b * p.q_len; }
 __device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) {
@@ -72,7 +80,7 @@ __device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) {
     if (ql <= 0) return 0;  // no query rows: nothing to compute, the sequence contributes no tile
     if (p.len_excludes_new) len += ql;
   }
-  return len;
+  return min(max(len, 0), p.max_len);
 }
 
 // Number of KV splits of one sequence and the (tile-aligned) tokens per split, generic kernel.
@@ -95,6 +103,9 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype);
 size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int batch);
 const char* launch_mfma(const DecodeParams& p, int q_dtype, int kv_dtype, bool skip_combine, hipStream_t s);
+// Compute units of the current device (256 on MI355X; that figure also when no device is visible, so that workspace
+// plans can be made on a host without a GPU).  Asked once per device.
+int device_cu_count();
 const char* launch_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
                                 void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size,
                                 int64_t n_pages, hipStream_t s);

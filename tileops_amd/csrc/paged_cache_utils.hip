@@ -5,14 +5,17 @@
 namespace mi355 {
 
 // One workgroup per (logical token, sequence): copy the physical row the block table names into the
-// dense [batch, max_len, row_bytes] output.  Uses physical_token(), the page arithmetic shared with the
-// attention kernels, so a bit-exact comparison against torch indexing pins that arithmetic.
+// dense [batch, max_len, row_bytes] output.  Uses physical_token(), the page arithmetic of the generic attention
+// kernel and of the append kernels below, so a bit-exact comparison against torch indexing pins that arithmetic.
+// (The MFMA attention kernel walks the table with its own incremental cursor; its gather is pinned bit-exactly by a
+// test that makes one key dominant and reads the physical row id back out of the attention output.)
 __global__ void gather_probe_kernel(const uint32_t* __restrict__ cache, const int32_t* __restrict__ seqlens,
                                     const int32_t* __restrict__ block_table, int64_t bt_row_stride,
                                     uint32_t* __restrict__ dense_out, int64_t max_len, int64_t row_dwords,
                                     int page_size, int64_t n_pages) {
   const int b = blockIdx.y;
-  const int len = seqlens[b];
+  const int64_t cap = bt_row_stride * (int64_t)page_size;  // what the sequence's block-table row can address
+  const int64_t len = seqlens[b] < cap ? seqlens[b] : cap;
   for (int64_t t = blockIdx.x; t < len && t < max_len; t += gridDim.x) {
     const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, (int)t, page_size, n_pages);
     const uint32_t* src = cache + phys * row_dwords;
@@ -41,7 +44,7 @@ __global__ __launch_bounds__(64) void kv_append_fp8_kernel(const uint16_t* __res
                                                            int heads_kv, int dim, int page_size, int64_t n_pages) {
   const int b = blockIdx.y, kvh = blockIdx.x, lane = threadIdx.x;
   const int len = seqlens[b];
-  if (len <= 0) return;
+  if (len <= 0 || (len - 1) / page_size >= bt_row_stride) return;  // a position the block-table row cannot address: write nothing
   const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, len - 1, page_size, n_pages);
   const uint16_t* xp = x_new + ((int64_t)b * heads_kv + kvh) * dim;
   const int per = dim / 64 > 0 ? dim / 64 : 1;  // dim in {64,128,256}: 1, 2 or 4 elements per lane, consecutive
@@ -109,6 +112,7 @@ __global__ __launch_bounds__(256) void kv_append_chunk_kernel(const uint16_t* __
   const int b = lo;
   if (t >= cu_q[b + 1]) return;
   const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
+  if (pos < 0 || pos / page_size >= bt_row_stride) return;  // a position the block-table row cannot address: write nothing
   const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages);
   const uint16_t* ks = k_new + t * row_elems;
   const uint16_t* vs = v_new + t * row_elems;
@@ -190,6 +194,7 @@ __global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* 
   const int b = lo;
   if (t >= cu_q[b + 1]) return;
   const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
+  const bool addressable = pos >= 0 && pos / page_size < bt_row_stride;  // else: rotate the query, append nothing
   const int64_t tpos = pos < max_position ? pos : max_position - 1;  // the caller checks positions; never read past the tables
   const int half = rotary_dim >> 1;
   const uint16_t* cs = cos_table + tpos * half;
@@ -204,7 +209,7 @@ __global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* 
   const int64_t q_elems = (int64_t)heads * dim, kv_elems = (int64_t)heads_kv * dim;
   const uint16_t* qs = q + t * q_elems;
   uint16_t* qd = q_rot + t * q_elems;
-  const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages);
+  const int64_t phys = addressable ? physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages) : 0;
   const uint16_t* ks = k_new + t * kv_elems;
   const uint16_t* vs = v_new + t * kv_elems;
   uint16_t* kd = k_pages + phys * kv_elems;
@@ -239,6 +244,7 @@ __global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* 
       const int h = i / items, it = i - h * items;
       head_item(qs + (int64_t)h * dim, qd + (int64_t)h * dim, it);
     }
+    if (!addressable) return;
     for (int i = threadIdx.x; i < heads_kv * items; i += 256) {
       const int h = i / items, it = i - h * items;
       head_item(ks + (int64_t)h * dim, kd + (int64_t)h * dim, it);
@@ -250,6 +256,7 @@ __global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* 
     const int d = (int)(i % dim);
     qd[i] = rotate(qs + (i - d), d);
   }
+  if (!addressable) return;
   for (int64_t i = threadIdx.x; i < kv_elems; i += 256) {
     const int d = (int)(i % dim);
     kd[i] = rotate(ks + (i - d), d);

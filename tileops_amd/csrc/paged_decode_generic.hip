@@ -64,8 +64,8 @@ __global__ __launch_bounds__(256) void paged_decode_generic_kernel(const DecodeP
     bool valid = r < rows_b;
     int s = valid ? r / p.group : 0, gidx = valid ? r % p.group : 0;
     const char* qp = (const char*)p.q + (((q_row0 + s) * p.heads + kvh * p.group + gidx) * D + c * EPL) * QB;
-    uint32_t raw[EPL * QB / 4];
-    load_raw<EPL * QB>(qp, raw);
+    uint32_t raw[EPL * QB / 4] = {};
+    if (valid) load_raw<EPL * QB>(qp, raw);  // a row past the sequence's own rows may lie past the end of q
     Unpack<QT, EPL>::run(raw, qf[rr]);
     limit[rr] = valid ? ((p.causal && p.q_len > 1) ? len - q_len_b + s + 1 : len) : 0;
   }

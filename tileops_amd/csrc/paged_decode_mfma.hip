@@ -28,6 +28,8 @@
 //    row split into two e4m3fn rows (hi + lo, exact for bf16 queries); at head dim 64 K is widened like V.
 //    The per-token K scale multiplies the score and the V scale multiplies the probability, so no
 //    head_dim-wide multiplies are spent on dequantisation.  Scales ride the same direct-to-LDS pipeline.
+#include <atomic>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -48,7 +50,6 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 constexpr int kCT = 32;       // tokens per pipeline stage (one MFMA K-block of the PV product)
 constexpr int kD = 128;       // default head dim (64 and 256 also run)
-constexpr int kNumCU = 256;   // MI355X
 // Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
 constexpr bool kLateIssueNarrow = true;
@@ -268,10 +269,6 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   const int wave = uni(threadIdx.x >> 6);
   // Workgroups are dealt round-robin to the 8 XCDs, so neighbouring partitions (which read neighbouring pages of
   // a sequence) spread over all L2s and memory channels; renumbering them XCD-contiguously measured slower.
-#ifdef MI355_PHASE_TIMERS
-  const uint64_t tm_kernel0 = __builtin_readcyclecounter();
-  const uint64_t tm_wall0 = wall_clock64();  // constant 100 MHz, common to all XCDs (the cycle counter is per XCD clock)
-#endif
   const int gw = blockIdx.x * NW + wave;
   const int n_rg = ring_row_groups(p.rows, NRB, SHW);
   const int per_part = p.heads_kv * n_rg;
@@ -919,39 +916,24 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       return score_step((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
     }
   };
-#ifdef MI355_PHASE_TIMERS
-  // Measurement build only (-DMI355_PHASE_TIMERS, see tileops_amd/perf/phase_timers.py): per-wave cycle totals of the
-  // loop phases and wall-clock start/end stamps, eight floats per wave written behind the workspace proper.
-  uint64_t tm_issue = 0, tm_wait = 0, tm_comp = 0, tm_seg = 0, tm_mark = __builtin_readcyclecounter();
-  const uint64_t tm_loop0 = tm_mark;
-  // (the scheduling barriers keep the compiler from moving vector work of one phase across the stamp of the next)
-#define TM(acc) { __builtin_amdgcn_sched_barrier(0); uint64_t now_ = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); acc += now_ - tm_mark; tm_mark = now_; }
-#else
-#define TM(acc)
-#endif
   int u = 0, ring = 0, seg_count = 0;
   while (u < n_units) {
     const int seg_first_j = cc.j;
     const int seg_units = min(cc.nt - cc.j, n_units - u);
     if (!LATE) issue_ahead(ring);  // before the query loads, so the next tile is already in flight while they land
-    TM(tm_issue)
     begin_segment(cc);
-    TM(tm_seg)
     int k = 0;
     while (k < seg_units) {
       bool moved = false;
       for (; k < seg_units; ++k) {  // steady state: no tile in here rescales the accumulators
         if (!LATE && k > 0) issue_ahead(ring);
-        TM(tm_issue)
         wait_stage(u);
         if (SH) {
           // Own part of tile u has landed; past the barrier so have the others', and every wave of the workgroup
           // has finished reading tile u-1, whose slot the next fetch overwrites.
           asm volatile("s_barrier" ::: "memory");
         }
-        TM(tm_wait)
         if (LATE) issue_ahead(ring);
-        TM(tm_issue)
         moved = run_score_step(ring);
         if constexpr ((SH && D <= 128) || (FP8 && NRB == 2)) {
           // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
@@ -961,7 +943,6 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
           if (__builtin_expect(moved, 0)) break;
         }
         value_step();
-        TM(tm_comp)
         ++u;
         ++cc.j;
         ring = ring + 1 == NS ? 0 : ring + 1;
@@ -969,7 +950,6 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
       if (moved) {  // rare after the first tiles of a sequence: finish this tile out of line, then re-enter
         rescale();
         value_step();
-        TM(tm_comp)
         ++u;
         ++cc.j;
         ring = ring + 1 == NS ? 0 : ring + 1;
@@ -980,17 +960,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
     end_segment(cc, seg_first_j == 0 && cc.j == cc.nt - 1, seg_count == 0 ? 0 : 1);
     ++seg_count;
     cursor_next(cc, p, ps16);
-    TM(tm_seg)
   }
-#ifdef MI355_PHASE_TIMERS
-  if (lane == 0) {
-    float* dst = (float*)(ws_prefix + ((p.batch + 1) * 4 + 63) / 64 * 64) + (size_t)gw * 8;  // past the records: caller over-allocates
-    dst[0] = (float)tm_issue; dst[1] = (float)tm_wait; dst[2] = (float)tm_comp; dst[3] = (float)tm_seg;
-    dst[4] = (float)(tm_loop0 - tm_kernel0); dst[5] = (float)(tm_mark - tm_kernel0);
-    dst[6] = (float)(tm_wall0 & 0xFFFFFF); dst[7] = (float)(wall_clock64() & 0xFFFFFF);
-  }
-#endif
-#undef TM
 }
 
 // Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
@@ -1286,13 +1256,13 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   const size_t lds = (size_t)(SH ? 1 : NW) * NS * Geom<KVT, D>::STAGE;
   auto kern = paged_decode_mfma_kernel<QT, KVT, NRB, NS, NW, SHW, D>;
   // the LDS opt-in is a per-device function attribute: set once per device, not on every launch
-  static bool lds_opted_in[64] = {};  // (one flag array per instantiation)
+  static std::atomic<bool> lds_opted_in[64];  // (one flag array per instantiation; zero-initialised)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return "hipGetDevice failed";
-  if (dev < 0 || dev >= 64 || !lds_opted_in[dev]) {
+  if (dev < 0 || dev >= 64 || !lds_opted_in[dev].load(std::memory_order_acquire)) {
     hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e0 != hipSuccess) return hipGetErrorString(e0);
-    if (dev >= 0 && dev < 64) lds_opted_in[dev] = true;
+    if (dev >= 0 && dev < 64) lds_opted_in[dev].store(true, std::memory_order_release);  // (setting it twice from two threads is harmless)
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, s, p, ws_prefix);
   hipError_t e = hipGetLastError();
@@ -1384,7 +1354,7 @@ int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
   const int waves_per_cu = dim == 256 ? ((shw > 1 || fp8) ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
-  const int64_t waves = (int64_t)kNumCU * waves_per_cu;
+  const int64_t waves = (int64_t)device_cu_count() * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
 }

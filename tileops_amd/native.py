@@ -19,7 +19,7 @@ ABI_VERSION = 1
 
 DT_BF16, DT_FP16, DT_FP8_E4M3FN = 0, 1, 2
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
-KERNEL_FLAG_SKIP_COMBINE = 0x100  # measurement aid: attention kernel only, partials left unmerged
+KERNEL_FLAG_SKIP_COMBINE = 0x100  # this package's benchmark only (csrc/common.h): attention kernel alone, partials left unmerged
 KERNEL_NAMES = {KERNEL_AUTO: "auto", KERNEL_GENERIC: "generic", KERNEL_MFMA: "mfma"}
 
 EXPORTED_SYMBOLS = (
