@@ -112,6 +112,60 @@ def _prop(value: Any) -> str:
     return str(value)
 
 
+_NOT_A_MEASUREMENT = frozenset({"tag", "op", "op_module"})  # set by the recorder, not measured
+
+
+def junit_case(suite: ET.Element, name: str, entries: list[dict]) -> ET.Element:
+    """One ``<testcase>`` with the properties the reference's pytest hook attaches (benchmarks/conftest.py:52-136).
+
+    ``entries`` are the records of one benchmark case, each ``{"tag", "op", "op_module", <measurements>}``.  The first
+    entry whose tag starts with ``tileops`` gives ``op``, ``op_module``, ``tileops_variant`` (for a tag
+    ``tileops_<variant>``) and ``tileops_<metric>``; every other entry is written under its own tag as
+    ``<tag>_<metric>``, the first of them also as ``baseline_<metric>`` with ``baseline_tag``; ``<tag>_ratio`` (and
+    ``baseline_ratio``) = baseline time over ours, on ``device_busy_ms`` when both sides have it, else on ``latency_ms``.
+    ``None`` values are left out.
+    """
+    ours = next((e for e in entries if e["tag"].startswith("tileops")), None)
+    baselines = [e for e in entries if not e["tag"].startswith("tileops")]
+    lat = (ours or {}).get("latency_ms") or 0.0
+    case = ET.SubElement(suite, "testcase", classname=(ours or entries[0]).get("op", ""), name=name, time=f"{lat / 1e3:.6f}")
+    props = ET.SubElement(case, "properties")
+
+    def emit(tag: str, entry: dict) -> None:
+        for key, val in entry.items():
+            if key in _NOT_A_MEASUREMENT or val is None:
+                continue
+            ET.SubElement(props, "property", name=f"{tag}_{key}", value=_prop(val))
+
+    if ours:
+        ET.SubElement(props, "property", name="op", value=ours["op"])
+        if "op_module" in ours:
+            ET.SubElement(props, "property", name="op_module", value=ours["op_module"])
+        tag = ours["tag"]
+        if tag != "tileops" and tag.startswith("tileops_"):
+            ET.SubElement(props, "property", name="tileops_variant", value=tag[len("tileops_"):])
+        emit("tileops", ours)
+    for idx, be in enumerate(baselines):
+        emit(be["tag"], be)
+        if idx == 0:
+            ET.SubElement(props, "property", name="baseline_tag", value=be["tag"])
+            emit("baseline", be)
+        if not ours:
+            continue
+        key = "device_busy_ms" if (ours.get("device_busy_ms") or 0) > 0 and (be.get("device_busy_ms") or 0) > 0 else "latency_ms"
+        tl, bl = ours.get(key) or 0, be.get(key) or 0
+        if tl > 0 and bl > 0:
+            ET.SubElement(props, "property", name=f"{be['tag']}_ratio", value=f"{bl / tl:.4f}")
+            if idx == 0:
+                ET.SubElement(props, "property", name="baseline_ratio", value=f"{bl / tl:.4f}")
+    return case
+
+
+def write_junit(suite: ET.Element, path: Path) -> None:
+    suite.set("tests", str(len(suite.findall("testcase"))))
+    ET.ElementTree(suite).write(path, encoding="utf-8", xml_declaration=True)
+
+
 class _Flusher:
     """Evicts L2 and the memory-side cache between timed calls: a 512 MiB write followed by a 512 MiB read."""
 
@@ -321,31 +375,21 @@ def main(argv: Optional[list[str]] = None) -> int:
                 if "page_size" in row:
                     params["page_size"] = row["page_size"]
                 report.record(op_name, params, res, "tileops", getattr(kernel, "config", None))
-                case = ET.SubElement(suite, "testcase", classname=op_name, name=f"{row['label']}-{dname}", time=f"{lat / 1e3:.6f}")
-                props = ET.SubElement(case, "properties")
-                ET.SubElement(props, "property", name="op", value=op_name)
-                ET.SubElement(props, "property", name="op_module", value=type(op).__module__)
-                for key, val in res.items():
-                    ET.SubElement(props, "property", name=f"tileops_{key}", value=_prop(val))
+                entries = [dict(res, tag="tileops", op=op_name, op_module=type(op).__module__)]
                 line = f"{op_name[:40]:40s} {row['label']:28s} {dname:9s} {lat * 1e3:9.1f} us  {res['bandwidth_tbs']:.2f} TB/s ({100 * res['hbm_frac']:.1f}%)"
                 if baseline is not None:
                     bl = _time(baseline, flush, max(args.steps // 2, 3))
                     flops, nbytes = op.eval_roofline()
                     bres = {"latency_ms": bl, "tflops": flops / bl / 1e9, "bandwidth_tbs": nbytes / bl / 1e9}
                     report.record(op_name, params, bres, "torch_sdpa")
-                    ET.SubElement(props, "property", name="baseline_tag", value="torch_sdpa")
-                    for key, val in bres.items():
-                        ET.SubElement(props, "property", name=f"torch_sdpa_{key}", value=_prop(val))
-                        ET.SubElement(props, "property", name=f"baseline_{key}", value=_prop(val))
-                    ET.SubElement(props, "property", name="torch_sdpa_ratio", value=f"{bl / lat:.4f}")
-                    ET.SubElement(props, "property", name="baseline_ratio", value=f"{bl / lat:.4f}")
+                    entries.append(dict(bres, tag="torch_sdpa", op=op_name))
                     line += f"   torch_sdpa {bl * 1e3:9.1f} us (x{bl / lat:.2f})"
+                junit_case(suite, f"{row['label']}-{dname}", entries)
                 print(line, flush=True)
                 n += 1
                 del op, inputs, baseline, call
                 torch.cuda.empty_cache()
-    suite.set("tests", str(n))
-    ET.ElementTree(suite).write(out_dir / "junit.xml", encoding="utf-8", xml_declaration=True)
+    write_junit(suite, out_dir / "junit.xml")
     report.dump(out_dir / "profile_run.log")
     print(f"{n} workloads -> {out_dir}/junit.xml, {out_dir}/profile_run.log")
     return 0
