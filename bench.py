@@ -1,10 +1,13 @@
 """Headline benchmark: paged GQA decode on one MI355X.
 
 One "step" = one forward of the op over one batch of synthetic input already resident in HBM.  Prints ONE JSON
-line: us/call of the Llama-3-8B-shape bf16 configuration (BASELINE config 2) with the HBM roofline of the call,
-the CPU oracle timed on this box's host cores beside it, and (in ``also``) the FP8-KV configuration.
+line: us/call of the Llama-3-8B-shape bf16 configuration (config 2) with the HBM roofline of its dominant kernel and the
+CPU references timed on this box's host cores beside it; ``also`` holds the same blocks for the FP8-KV configuration
+(c3), the 8 x 128K-token split-KV configuration (c4) and the eight-query-token configuration (c5).  The four
+configurations are workload rows of the op manifest (``load_workloads``); bytes and flops come from the op's
+``eval_roofline()`` after it has seen the call.  Exit status 1 if any configuration misses its parity tolerance.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--also c3,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--also c3,c4,c5] [--no-cpu]
 """
 
 from __future__ import annotations
@@ -21,17 +24,54 @@ ROOT = Path(__file__).resolve().parent
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
-HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense bf16 matrix rate (the PV product and, for 16-bit caches, QK^T run in bf16)
+TRAFFIC_SOURCE = "profiles/hbm_traffic.json"
+
+DESCRIPTIONS = {
+    "c2": "Llama-3-8B-shape paged GQA decode, bf16 KV",
+    "c3": "Llama-3-8B-shape paged GQA decode, FP8-e4m3fn KV with per-token scales",
+    "c4": "long-context split-KV stress, 8 x 131072 tokens, FP8 KV",
+    "c5": "multi-token (speculative verify) decode, 8 query tokens, FP8 KV",
+}
+
+
+def _config(name: str):
+    """The configuration as the manifest states it."""
+    from tileops_amd.manifest import load_workloads
+    from tileops_amd.workloads import BASELINE_WORKLOAD_ROWS, config_from_workload
+
+    op_name, label = BASELINE_WORKLOAD_ROWS[name]
+    row = next(r for r in load_workloads(op_name) if r["label"] == label)
+    return config_from_workload(row, name, DESCRIPTIONS[name]), op_name, label
+
+
+def _timed_steps(fn, flush, steps: int) -> tuple[list[float], float]:
+    """``steps`` calls, each after a cache flush and between its own pair of events on the stream the kernels run on."""
+    import torch
+
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    for i in range(steps):
+        flush(i)
+        starts[i].record()
+        fn()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    return [s.elapsed_time(e) for s, e in zip(starts, stops)], wall
 
 
 def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: str | None) -> dict:
     import torch
 
     from tileops_amd import ops
-    from tileops_amd.roofline import algorithmic_bytes, algorithmic_flops
-    from tileops_amd.workloads import BASELINE_CONFIGS, gen_paged_inputs
+    from tileops_amd.roofline import algorithmic_bytes
+    from tileops_amd.workloads import gen_paged_inputs
 
-    cfg = BASELINE_CONFIGS[name]
+    cfg, op_name, label = _config(name)
     device = torch.device("cuda", 0)
     inp = gen_paged_inputs(cfg, device)
     if cfg.q_len == 1:
@@ -39,32 +79,26 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     else:
         op = ops.GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp(cfg.batch, cfg.q_len, cfg.heads, cfg.heads_kv, cfg.seqlen_kv,
                                                                             cfg.dim, cfg.page_size)
+    assert type(op).__name__ == op_name
     if kernel_key:
         op.kernel_map = {kernel_key: op.kernel_map[kernel_key]}
     args = inp.as_args()
     # Between steps a 512 MiB buffer is overwritten and a second 512 MiB buffer is read: the write evicts L2 and
     # the 256 MB Infinity Cache, the read pushes the dirty lines out again so the timed call starts on a clean,
     # cold cache and every K/V byte comes from HBM.
-    flush = torch.empty(512 << 20, dtype=torch.uint8, device=device)
+    flush_wr = torch.empty(512 << 20, dtype=torch.uint8, device=device)
     flush_rd = torch.ones(128 << 20, dtype=torch.int32, device=device)
+
+    def flush(i: int) -> None:
+        flush_wr.fill_(i & 0xFF)
+        flush_rd.max()
+
     for _ in range(max(warmup, 1)):
         out = op(*args)
     torch.cuda.synchronize()
-    # timed region: exactly `steps` calls, each bracketed by events on the stream the kernels run on
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    torch.cuda.synchronize()
-    wall0 = time.perf_counter()
-    for i in range(steps):
-        flush.fill_(i & 0xFF)
-        flush_rd.max()
-        starts[i].record()
-        out = op(*args)
-        stops[i].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    per_step_ms = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+    per_step_ms, wall = _timed_steps(lambda: op(*args), flush, steps)
     ms = sum(per_step_ms) / steps
+    ms_median = statistics.median(per_step_ms)
     # the same K calls back to back (no flush) for reference
     s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s0.record()
@@ -74,87 +108,124 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     torch.cuda.synchronize()
     b2b_ms = s0.elapsed_time(s1) / steps
 
-    # The dominant (attention) kernel alone: launches that skip the combine kernel, KREP back to back per event
-    # pair so that the few microseconds an event pair costs are spread over KREP launches.  Each launch streams
+    # The dominant (attention) kernel alone: launches that skip the merge of partial results, KREP back to back per
+    # event pair so that the few microseconds an event pair costs are spread over KREP launches.  Each launch streams
     # far more than the 256 MB Infinity Cache holds, so a launch finds next to nothing of its predecessor cached.
     KREP = 4
     kernel = next(iter(next(iter(op._kernel_roles.values())).values()))
     kernel.attention_kernel_only = True
-    k_starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    k_stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for i in range(steps):
-        flush.fill_(i & 0xFF)
-        flush_rd.max()
-        k_starts[i].record()
+
+    def attention_only() -> None:
         for _ in range(KREP):
             op(*args)
-        k_stops[i].record()
-    torch.cuda.synchronize()
-    kernel.attention_kernel_only = False
-    kernel_ms = sum(s.elapsed_time(e) for s, e in zip(k_starts, k_stops)) / (steps * KREP)
-    out = op(*args)  # complete output again for the parity check below
 
+    k_ms, _ = _timed_steps(attention_only, flush, steps)
+    kernel.attention_kernel_only = False
+    kernel_ms = sum(k_ms) / (steps * KREP)
+    out = op(*args)  # complete output again for the parity check below
+    torch.cuda.synchronize()
+
+    # a whole call captured once in a HIP graph and replayed (what a serving loop does): no host launch gaps
+    graph_ms = graph_median_ms = None
+    if hasattr(op, "capture"):
+        replay = op.capture(*args)
+        for _ in range(3):
+            replay()
+        g_ms, _ = _timed_steps(replay, flush, steps)
+        graph_ms, graph_median_ms = sum(g_ms) / steps, statistics.median(g_ms)
+        torch.cuda.synchronize()
+
+    op.observe_call(inp.real_seqlen_kv, cfg.kv_dtype)
+    flops, total_bytes = op.eval_roofline()
     lens = inp.real_seqlen_kv.cpu().to(torch.int64)
     sum_len = int(lens.sum())
     sum_pages = int(((lens + cfg.page_size - 1) // cfg.page_size).sum())
     fp8 = cfg.kv_dtype == torch.float8_e4m3fn
     b = algorithmic_bytes(sum_len=sum_len, sum_pages=sum_pages, batch=cfg.batch, q_len=cfg.q_len, heads=cfg.heads, heads_kv=cfg.heads_kv,
                           dim=cfg.dim, q_bytes=2, kv_bytes=1 if fp8 else 2, fp8_scales=fp8)
-    flops = algorithmic_flops(sum_len=sum_len, q_len=cfg.q_len, heads=cfg.heads, dim=cfg.dim)
-    achieved = b["total"] / (kernel_ms * 1e-3) / 1e9
+    assert b["total"] == total_bytes
+    kv_read = b["kv"] + b["scales"]
+    achieved = total_bytes / (kernel_ms * 1e-3) / 1e9
     traffic = None
-    try:  # measured with hardware counters in a separate profiler run; absent for configurations not profiled
-        traffic = json.loads((ROOT / "profiles" / "hbm_traffic.json").read_text()).get(name, {}).get("traffic_bytes")
+    try:  # measured with hardware counters in a separate profiler run (not in this run); absent for configurations not profiled
+        traffic = json.loads((ROOT / TRAFFIC_SOURCE).read_text()).get(name, {}).get("traffic_bytes")
     except (OSError, ValueError):
         pass
+
+    def gbs(nbytes: int, t_ms: float) -> float:
+        return nbytes / (t_ms * 1e-3) / 1e9
+
     res = {
-        "workload": f"{name}: {cfg.description}; batch {cfg.batch}, q_len {cfg.q_len}, {cfg.heads}q/{cfg.heads_kv}kv heads, dim {cfg.dim}, "
-                    f"page {cfg.page_size}, len in {list(cfg.len_range)}, {cfg.n_pages}-page pool, seed {cfg.seed}",
+        "workload": f"{name} = manifest row '{label}': {cfg.description}; batch {cfg.batch}, q_len {cfg.q_len}, {cfg.heads}q/{cfg.heads_kv}kv heads, "
+                    f"dim {cfg.dim}, page {cfg.page_size}, len in {list(cfg.len_range)}, {cfg.n_pages}-page pool, seed {cfg.seed}",
         "kernel": type(kernel).__name__,
         "us_per_call": ms * 1e3,
-        "us_per_call_median": statistics.median(per_step_ms) * 1e3,
+        "us_per_call_median": ms_median * 1e3,
         "us_per_call_back_to_back": b2b_ms * 1e3,
         "sum_len": sum_len,
         "decode_tokens_per_s": cfg.batch * cfg.q_len / (ms * 1e-3),
         "kv_tokens_per_s": sum_len / (ms * 1e-3),
         "algorithmic_bytes": b,
         "flops": flops,
-        "kv_read_gbs": (b["kv"] + b["scales"]) / (ms * 1e-3) / 1e9,
+        # the whole call (attention kernel, merge of partial results where one is launched, launch gaps): mean and median of the
+        # flushed steps, on the K/V (+ scale) bytes alone -- the figure the 70 % target is stated on -- and on all bytes
+        "whole_call": {
+            "us_mean": ms * 1e3, "us_median": ms_median * 1e3,
+            "kv_read_gbs_mean": gbs(kv_read, ms), "kv_read_gbs_median": gbs(kv_read, ms_median),
+            "kv_read_frac_of_peak_mean": gbs(kv_read, ms) / HBM_PEAK_GBS, "kv_read_frac_of_peak_median": gbs(kv_read, ms_median) / HBM_PEAK_GBS,
+            "all_bytes_frac_of_peak_mean": gbs(total_bytes, ms) / HBM_PEAK_GBS,
+        },
         "attention_kernel_us": kernel_ms * 1e3,
-        "whole_call_gbs": b["total"] / (ms * 1e-3) / 1e9,
-        "whole_call_frac_of_peak": b["total"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        # dominant kernel: algorithmic bytes of one launch / its own duration (events around the attention kernel alone)
+        # dominant kernel alone: algorithmic bytes of one launch / its own duration (events around the attention kernel only)
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic},
+                     "traffic": traffic, "traffic_source": f"{TRAFFIC_SOURCE} (rocprofv3 FETCH_SIZE/WRITE_SIZE of an earlier profiler run, not counted in this run)"},
         "wall_s_timed_region": wall,
     }
+    if graph_ms is not None:
+        res["whole_call"].update({
+            "us_graph_mean": graph_ms * 1e3, "us_graph_median": graph_median_ms * 1e3,
+            "kv_read_frac_of_peak_graph_mean": gbs(kv_read, graph_ms) / HBM_PEAK_GBS,
+            "kv_read_frac_of_peak_graph_median": gbs(kv_read, graph_median_ms) / HBM_PEAK_GBS,
+        })
+    if cfg.q_len * (cfg.heads // cfg.heads_kv) >= 16:
+        # enough query rows per kv head for the products to be dense matrix work: report the matrix rate beside the bandwidth
+        tf = flops / (kernel_ms * 1e-3) / 1e12
+        res["mfma"] = {"flops": flops, "achieved_tflops": tf, "peak_tflops": MFMA_PEAK_TFLOPS, "frac_of_2500": tf / MFMA_PEAK_TFLOPS}
     if with_cpu:
-        from oracle.paged_gqa_decode_ref import ref_paged_gqa_decode
+        from oracle.paged_gqa_decode_ref import ref_paged_gqa_decode, ref_paged_gqa_decode_sdpa_math
 
         host = inp.to("cpu")
         threads = os.cpu_count() or 1
         torch.set_num_threads(threads)
         kw = dict(page_size=cfg.page_size, k_scale=host.k_scale, v_scale=host.v_scale)
-        # bounded sample: as many leading sequences as take roughly 10 s, timed 3 times (median)
+        # bounded sample: as many leading sequences as take roughly 6 s, timed 3 times (median)
         t0 = time.perf_counter()
         ref_paged_gqa_decode(host.q[:1], host.k, host.v, host.real_seqlen_kv[:1], host.block_table[:1], **kw)
         one = time.perf_counter() - t0
-        n_seq = max(1, min(cfg.batch, int(10.0 / max(one, 1e-3))))
+        n_seq = max(1, min(cfg.batch, int(6.0 / max(one, 1e-3))))
         times = []
         for _ in range(3):
             t0 = time.perf_counter()
             ref = ref_paged_gqa_decode(host.q[:n_seq], host.k, host.v, host.real_seqlen_kv[:n_seq], host.block_table[:n_seq], **kw)
             times.append(time.perf_counter() - t0)
         sample_len = int(lens[:n_seq].sum())
-        cpu_s = statistics.median(times) * (sum_len / sample_len)  # scaled to the whole batch by tokens
+        scale_up = sum_len / sample_len
+        cpu_s = statistics.median(times) * scale_up  # scaled to the whole batch by tokens
+        t0 = time.perf_counter()
+        ref_sdpa = ref_paged_gqa_decode_sdpa_math(host.q[:n_seq], host.k, host.v, host.real_seqlen_kv[:n_seq], host.block_table[:n_seq], **kw)
+        sdpa_s = (time.perf_counter() - t0) * scale_up
         tol = 3e-2 if fp8 else 2e-2
-        err = (out[:n_seq].float().cpu() - ref.float()).abs().max().item()
-        ok = torch.allclose(out[:n_seq].float().cpu(), ref.float(), atol=tol, rtol=tol)
+        got = out[:n_seq].float().cpu()
+        err = (got - ref.float()).abs().max().item()
+        ok = torch.allclose(got, ref.float(), atol=tol, rtol=tol) and torch.allclose(got, ref_sdpa.float(), atol=tol, rtol=tol)
+        sample = f"the first {n_seq} of {cfg.batch} sequences ({sample_len} of {sum_len} KV tokens), scaled by tokens to the whole batch"
         res["cpu_baseline"] = {"value": cpu_s * 1e6, "unit": "us/call", "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"torch fp32 oracle on the first {n_seq} of {cfg.batch} sequences ({sample_len} of {sum_len} KV tokens), "
-                                         f"median of 3 runs, scaled by tokens to the whole batch"}
+                               "sample": f"torch fp32 oracle (gather pages, dequantise, grouped einsum softmax) on {sample}, median of 3 runs"}
+        res["cpu_baseline_sdpa_math"] = {"value": sdpa_s * 1e6, "unit": "us/call", "cores": torch.get_num_threads(), "kind": "port",
+                                         "sample": f"F.scaled_dot_product_attention under sdpa_kernel(MATH), fp32, heads expanded by indexing "
+                                                   f"(the torch baseline of the reference's own benchmark) on {sample}, one run"}
         res["parity"] = {"max_abs_err": err, "tolerance": tol, "within_tolerance": bool(ok), "sequences_checked": n_seq}
-    del inp, args, flush, flush_rd
+    del inp, args, flush_wr, flush_rd
     torch.cuda.empty_cache()
     return res
 
@@ -165,8 +236,8 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4", "c5"])
-    ap.add_argument("--also", default="c3", help="comma-separated extra configurations reported under 'also' ('' for none)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    ap.add_argument("--also", default="c3,c4,c5", help="comma-separated extra configurations reported under 'also' ('' for none)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU reference legs (and with them the parity check)")
     ap.add_argument("--kernel", default=None, choices=[None, "gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel"])
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies, so a hardware-counter pass has a kernel of known traffic to scale by")
@@ -181,7 +252,7 @@ def main() -> None:
     native.require_gfx950(torch.device("cuda", 0))
     main_res = _run_config(a.config, a.steps, a.warmup, not a.no_cpu, a.kernel)
     also = [_run_config(n, a.steps, a.warmup, not a.no_cpu, a.kernel) for n in a.also.split(",") if n and n != a.config]
-    fp8 = "fp8" in main_res["workload"].lower() and a.config != "c2"
+    fp8 = a.config != "c2"
     line = {
         "metric": "GQA paged-decode us/call (achieved HBM GB/s and fraction of the 8 TB/s peak under 'roofline')",
         "value": main_res["us_per_call"], "unit": "us/call", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -190,10 +261,10 @@ def main() -> None:
         "data": "synthetic", "config": {"workload": main_res["workload"], "kernel": main_res["kernel"]},
         "roofline": main_res["roofline"],
     }
-    if "cpu_baseline" in main_res:
-        line["cpu_baseline"] = main_res["cpu_baseline"]
-        line["parity"] = main_res["parity"]
-    line["detail"] = {k: v for k, v in main_res.items() if k not in ("roofline", "cpu_baseline", "parity", "workload")}
+    for key in ("cpu_baseline", "cpu_baseline_sdpa_math", "parity", "mfma"):
+        if key in main_res:
+            line[key] = main_res[key]
+    line["detail"] = {k: v for k, v in main_res.items() if k not in ("roofline", "cpu_baseline", "cpu_baseline_sdpa_math", "parity", "mfma", "workload")}
     line["also"] = also
     if a.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
@@ -203,6 +274,9 @@ def main() -> None:
         torch.cuda.synchronize()
         line["copy_calibration"] = {"bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "launches": 3}
     print(json.dumps(line))
+    failed = [r["workload"].split(" ")[0] for r in [main_res, *also] if "parity" in r and not r["parity"]["within_tolerance"]]
+    if failed:
+        sys.exit(f"parity outside tolerance for {', '.join(failed)}")
 
 
 if __name__ == "__main__":

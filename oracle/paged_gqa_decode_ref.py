@@ -12,6 +12,7 @@ Parity status of each function (how it is pinned, without importing the referenc
 * ``ref_paged_gqa_decode``      pinned against ``torch.nn.functional.scaled_dot_product_attention`` (a library
                                 routine, the reference benchmark's own baseline), a float64 NumPy brute force,
                                 and closed forms (q=0 -> mean of V, len=1 -> V row, dominant key, softcap->inf).
+* ``ref_paged_gqa_decode_sdpa_math``  the reference benchmark's torch baseline; pinned against ``ref_paged_gqa_decode``.
 * ``ref_gqa_decode_contiguous`` pinned against SDPA and the paged oracle with an identity table.
 * ``quantize_kv_per_token``     pinned against the C codec in ``oracle/fp8_e4m3fn.c`` and torch's fp8 cast.
 * causal chunk mask             pinned by "query i of a chunk == single-token decode at length len-S_q+i+1".
@@ -126,6 +127,47 @@ def ref_paged_gqa_decode(
         o = torch.einsum("jgsn,njd->sjgd", probs, v_b)
         out[b] = o.reshape(S_q, H, D)
     out = out.to(out_dtype or q.dtype)
+    return out if multi else out.squeeze(1)
+
+
+def ref_paged_gqa_decode_sdpa_math(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor, block_table: torch.Tensor, *,
+    page_size: int, k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None, is_causal: bool = True,
+) -> torch.Tensor:
+    """The torch baseline the reference *benchmark* times (benchmarks/ops/attention/bench_gqa_decode_paged.py:21-66):
+    per sequence, reassemble the pages, expand K/V to the query heads by indexing, and call
+    ``F.scaled_dot_product_attention`` under ``sdpa_kernel(MATH)`` -- in fp32 on the dequantized cache here, so that it
+    is the same function as ``ref_paged_gqa_decode`` (default scale, no softcap) computed by the library routine.
+    Multi-token queries pass the bottom-right causal mask explicitly.  Pinned against ``ref_paged_gqa_decode``."""
+    import torch.nn.functional as F
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    multi = q.dim() == 4
+    q4 = q if multi else q.unsqueeze(1)
+    B, S_q, H, D = q4.shape
+    H_kv = k.shape[1]
+    group_id = torch.arange(H, dtype=torch.long) // (H // H_kv)
+    out = torch.zeros(B, S_q, H, D, dtype=torch.float32)
+    for b in range(B):
+        n = int(real_seqlen_kv[b])
+        if n == 0:
+            continue
+        k_b = gather_pages(k, block_table[b], n, page_size).float()
+        v_b = gather_pages(v, block_table[b], n, page_size).float()
+        if k_scale is not None:
+            k_b = k_b * gather_pages(k_scale, block_table[b], n, page_size).float()[..., None]
+        if v_scale is not None:
+            v_b = v_b * gather_pages(v_scale, block_table[b], n, page_size).float()[..., None]
+        k_bhsd = k_b[:, group_id, :].unsqueeze(0).transpose(1, 2)
+        v_bhsd = v_b[:, group_id, :].unsqueeze(0).transpose(1, 2)
+        q_bhsd = q4[b].float().transpose(0, 1).unsqueeze(0)  # [1, H, S_q, D]
+        mask = None
+        if multi and is_causal and S_q > 1:
+            mask = torch.arange(n)[None, :] <= (torch.arange(S_q)[:, None] + (n - S_q))
+        with sdpa_kernel(backends=[SDPBackend.MATH]):
+            o = F.scaled_dot_product_attention(q_bhsd, k_bhsd, v_bhsd, attn_mask=mask)
+        out[b] = o[0].transpose(0, 1)
+    out = out.to(q.dtype)
     return out if multi else out.squeeze(1)
 
 

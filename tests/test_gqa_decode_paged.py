@@ -549,6 +549,66 @@ def test_graph_capture_and_replay_with_changing_cache_contents(fp8):
         assert torch.equal(eager, eager0) == (it == 0)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_op_capture_replays_equal_eager_calls(fp8):
+    """``op.capture(...)``: the whole call (attention and merge) recorded once in a HIP graph; every replay, with eager work and
+    synchronisation in between and new values, lengths and page ids written into the same tensors, equals the eager call."""
+    require_gfx950()
+    lens = [900, 33, 2048, 5, 1500, 64]
+    case = _ragged_case(len(lens), 32, 8, 128, 64, lens, torch.bfloat16, fp8=fp8, seed=19, poison=False)
+    dev = [None if t is None else t.to(DEV) for t in case]
+    args = dev[:5] if not fp8 else dev
+    op = PagedOp(len(lens), 32, 8, case[1].shape[0], 128, 64)
+    replay = op.capture(*args)
+    for it in range(4):
+        if it == 1:
+            args[2].mul_(-0.5) if not fp8 else args[6].mul_(1.5)          # new values in place
+        if it == 2:
+            args[3].copy_(torch.tensor([100, 33, 1024, 0, 1500, 1], dtype=torch.int32))   # shorter sequences, an empty one
+        if it == 3:
+            args[4][0, :4] = args[4][0, :4].flip(0)                        # other pages for the first 256 tokens of sequence 0
+        out_g = replay()
+        torch.cuda.synchronize()
+        eager = op(*args)
+        torch.cuda.synchronize()
+        assert torch.isfinite(eager).all()
+        assert torch.equal(out_g, eager), f"replay {it} differs from the eager call"
+
+
+@pytest.mark.parametrize("kernel_key", KERNELS)
+@pytest.mark.parametrize("fp8", [False, True])
+def test_lengths_are_clamped_to_what_the_block_table_row_addresses(kernel_key, fp8):
+    """A corrupt ``real_seqlen_kv`` -- far beyond the table's width, or negative -- must neither run a kernel past the
+    sequence's block-table row nor derail its neighbours: the oversized sequence computes exactly what it computes with
+    the length the row can address, the negative one what an empty one does (zeros), every other row is untouched, and
+    no unaddressed (NaN-filled) token is read.  The table sits inside a larger buffer whose other entries name a page
+    of NaNs, so a read past a row or past the table shows."""
+    require_gfx950()
+    page, width = 64, 4
+    lens_ok = [100, 0, width * page, 64, 200]
+    case = _ragged_case(len(lens_ok), 32, 8, 128, page, lens_ok, torch.bfloat16, fp8=fp8, seed=23)
+    q, k, v, lens, table, ks, vs = case
+    assert table.shape[1] == width
+    nan_page = int(table[1, 0])                      # the spare page unused entries name: all NaN
+    big = torch.full((len(lens_ok) + 2, width + 3), nan_page, dtype=torch.int32)
+    big[1:-1, :width] = table
+    dev = [None if t is None else t.to(DEV) for t in case]
+    dev[4] = big.to(DEV)[1:-1, :width]               # same values, row stride width + 3, NaN-page ids all around
+    op = PagedOp(len(lens_ok), 32, 8, k.shape[0], 128, page)
+    op.kernel_map = {kernel_key: op.kernel_map[kernel_key]}
+    args = dev[:5] if not fp8 else dev
+    want = op(*args).clone()
+    torch.cuda.synchronize()
+    assert torch.isfinite(want).all() and (want[1] == 0).all()
+    bad = torch.tensor([100, -7, 2 ** 31 - 1, 64, 200], dtype=torch.int32, device=DEV)
+    got = op(args[0], args[1], args[2], bad, *args[4:])
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    assert torch.equal(got, want)
+    bad2 = torch.tensor([100, -(2 ** 31), width * page + 1, 64, 200], dtype=torch.int32, device=DEV)
+    assert torch.equal(op(args[0], args[1], args[2], bad2, *args[4:]), want)
+
+
 def _random_configs(n, seed):
     """Seeded draw of small shapes over everything the ops accept: head counts and groups, head_dim, page size, query
     tokens, dtype, FP8 cache, softcap, custom scale (also negative), causal or not, ragged lengths with zeros."""

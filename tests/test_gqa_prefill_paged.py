@@ -347,6 +347,27 @@ def test_head_dims_64_and_256_with_chunks_of_hundreds_of_rows(dim, heads, heads_
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kernel", [native.KERNEL_GENERIC, native.KERNEL_AUTO], ids=["general", "mfma"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("heads, heads_kv", [(16, 4), (8, 8)])
+def test_fp8_cache_head_dim_256_like_the_qwen_fp8_row(kernel, dtype, heads, heads_kv):
+    """The reference's `qwen35-9b-prefill-paged-fp8-cache-b8-prefix32k-chunk1k-p64` row (attention.yaml:287: FP8 cache, head dim
+    256, page 64) at reduced sizes: 256-byte cache rows with per-tensor scales, the second pass over the chunk's own
+    16-bit tokens carrying the first pass's state.  A prefix that spans many partitions, an empty cache, an empty chunk,
+    a single-token chunk, a chunk that ends mid-page; on the general kernel and on the MFMA kernel."""
+    require_gfx950()
+    q_lens, old_lens = [257, 96, 0, 1, 40], [3000, 0, 100, 511, 333]
+    case = _case(q_lens, old_lens, heads, heads_kv, 256, dtype, fp8=True, page=64, max_pages=52, seed=29)
+    op = PrefillOp(batch=len(q_lens), heads=heads, heads_kv=heads_kv, max_pages_per_req=52, page_size=64, dim=256, cache_dtype=FP8)
+    call = op.attention_call(dtype, torch.device(DEV, 0))
+    key = op.select_kernel_key(tuple(op.kernel_map), call)
+    assert key == "gqa_prefill_paged_with_fp8_kv_cache_fwd_kernel"
+    inputs = [t.to(DEV) for t in case]
+    op._get_kernel(tuple(inputs), key, call).config["kernel"] = kernel
+    _run(op, case, 64, dtype, fp8=True)
+
+
+@pytest.mark.gpu
 def test_fused_rope_head_dim_256_partial_rotary_like_the_qwen_rows():
     """attention.yaml:280-281 at reduced size: head dim 256, rotary_dim 64, mixed chunk lengths against long prefixes."""
     require_gfx950()

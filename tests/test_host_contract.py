@@ -376,3 +376,20 @@ def test_entry_points_refuse_without_a_gfx950_device_before_launching():
     with pytest.raises(native.NativeLibraryError):
         native._check(lib.mi355_gather_probe(fake, fake, fake, 4, fake, 2, 256, 2048, 64, 64 * 8, None))
     assert "gfx950" in native.last_error() and q.device.type == "cpu"
+
+
+def test_benchmark_configurations_are_manifest_rows():
+    """bench.py takes its four GPU configurations from the manifest (`load_workloads`), not from shapes of its own: the
+    rows must describe exactly the configurations the parity tests run at full size."""
+    from tileops_amd.workloads import BASELINE_CONFIGS, BASELINE_WORKLOAD_ROWS, config_from_workload
+
+    assert set(BASELINE_WORKLOAD_ROWS) == set(BASELINE_CONFIGS) == {"c2", "c3", "c4", "c5"}
+    for name, (op_name, label) in BASELINE_WORKLOAD_ROWS.items():
+        row = next(r for r in load_workloads(op_name) if r["label"] == label)
+        want = BASELINE_CONFIGS[name]
+        assert config_from_workload(row, name, want.description) == want
+    for op_name in ("GroupedQueryAttentionDecodePagedWithKVCacheFwdOp", "GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp"):
+        entry = load_manifest()[op_name]
+        assert entry["source"]["bench"] == "bench.py" and entry["source"].get("bench_manifest_driven") is True
+    src = (ROOT / "bench.py").read_text()
+    assert "load_workloads(" in src and "eval_roofline()" in src

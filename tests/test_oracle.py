@@ -15,7 +15,7 @@ import torch.nn.functional as F
 
 from oracle.paged_gqa_decode_ref import (
     brute_force_f64, combine_partials, dequantize_kv, gather_pages, physical_pos, quantize_kv_per_token,
-    ref_gqa_decode_contiguous, ref_paged_gqa_decode, reference_block_ns, reference_roofline,
+    ref_gqa_decode_contiguous, ref_paged_gqa_decode, ref_paged_gqa_decode_sdpa_math, reference_block_ns, reference_roofline,
 )
 from tileops_amd.workloads import contiguous_as_paged, gen_contiguous_inputs
 
@@ -85,6 +85,23 @@ def test_matches_torch_sdpa_library_routine():
         vb = gather_pages(v, table[b], n, 8).repeat_interleave(4, dim=1).transpose(0, 1)
         want = F.scaled_dot_product_attention(q[b][:, None, :], kb, vb)[:, 0]
         torch.testing.assert_close(got[b], want, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("q_len", [1, 5])
+def test_sdpa_math_baseline_is_the_same_function_as_the_oracle(q_len):
+    """The reference benchmark's torch baseline (bench_gqa_decode_paged.py:21-66: reassemble pages, expand heads by index,
+    SDPA under the MATH backend) against the einsum oracle: ragged lengths, an empty sequence, FP8 with scales, and the
+    bottom-right causal mask for several query tokens."""
+    lens = [0 if q_len == 1 else q_len, 70, 129, 33]
+    q, k, v, lens_t, table = _case(4, 8, 2, 64, 32, lens, seed=5, q_len=q_len)
+    a = ref_paged_gqa_decode(q, k, v, lens_t, table, page_size=32)
+    b = ref_paged_gqa_decode_sdpa_math(q, k, v, lens_t, table, page_size=32)
+    torch.testing.assert_close(a, b, atol=2e-6, rtol=1e-5)
+    k8, ks = quantize_kv_per_token(k)
+    v8, vs = quantize_kv_per_token(v)
+    a = ref_paged_gqa_decode(q.bfloat16(), k8, v8, lens_t, table, page_size=32, k_scale=ks, v_scale=vs)
+    b = ref_paged_gqa_decode_sdpa_math(q.bfloat16(), k8, v8, lens_t, table, page_size=32, k_scale=ks, v_scale=vs)
+    torch.testing.assert_close(a.float(), b.float(), atol=1e-2, rtol=1e-2)  # both round an fp32 result to bf16
 
 
 def test_contiguous_reference_config1_and_identity_paging_agree():

@@ -64,6 +64,28 @@ BASELINE_CONFIGS: dict[str, PagedDecodeConfig] = {
 }
 
 
+#: Benchmark configuration name -> (op, label of its manifest workload row)
+BASELINE_WORKLOAD_ROWS: dict[str, tuple[str, str]] = {
+    "c2": ("GroupedQueryAttentionDecodePagedWithKVCacheFwdOp", "llama3-8b-paged-bf16"),
+    "c3": ("GroupedQueryAttentionDecodePagedWithKVCacheFwdOp", "llama3-8b-paged-fp8kv"),
+    "c4": ("GroupedQueryAttentionDecodePagedWithKVCacheFwdOp", "long-context-128k-fp8kv"),
+    "c5": ("GroupedQueryAttentionMultiTokenDecodePagedWithKVCacheFwdOp", "spec-verify-8tok-fp8kv"),
+}
+
+
+def config_from_workload(row: dict, name: str = "", description: str = "") -> PagedDecodeConfig:
+    """A manifest workload row with ``seqlen_range`` (ragged lengths over a shared pool, permuted block table) as a
+    ``PagedDecodeConfig``: ``q_shape`` ``[B, H, D]`` or ``[B, S_q, H, D]``, ``kv_shape`` ``[N_kv, H_kv, D]``."""
+    qs, (n_kv, heads_kv, dim) = list(row["q_shape"]), row["kv_shape"]
+    batch, heads = qs[0], qs[-2]
+    q_len = qs[1] if len(qs) == 4 else 1
+    dtype = getattr(torch, row["dtypes"][0])
+    kv_dtype = getattr(torch, row["kv_dtype"]) if row.get("kv_dtype") else dtype
+    page = row["page_size"]
+    return PagedDecodeConfig(name or row["label"], batch, heads, heads_kv, dim, page, n_kv // page, tuple(row["seqlen_range"]),
+                             q_len=q_len, dtype=dtype, kv_dtype=kv_dtype, seed=row.get("seed", 0), description=description)
+
+
 def quantize_kv_per_token(x: torch.Tensor, chunk_tokens: int = 1 << 16) -> tuple[torch.Tensor, torch.Tensor]:
     """``x [N, H_kv, D]`` -> (e4m3fn ``[N, H_kv, D]``, fp32 scale ``[N, H_kv]``): ``scale = max(absmax, 1e-4)/448``,
     ``q = clamp(x/scale, -448, 448)`` cast with round-to-nearest-even.  Chunked so a whole pool fits."""
