@@ -579,34 +579,27 @@ def test_op_capture_replays_equal_eager_calls(fp8):
 @pytest.mark.parametrize("fp8", [False, True])
 def test_lengths_are_clamped_to_what_the_block_table_row_addresses(kernel_key, fp8):
     """A corrupt ``real_seqlen_kv`` -- far beyond the table's width, or negative -- must neither run a kernel past the
-    sequence's block-table row nor derail its neighbours: the oversized sequence computes exactly what it computes with
-    the length the row can address, the negative one what an empty one does (zeros), every other row is untouched, and
-    no unaddressed (NaN-filled) token is read.  The table sits inside a larger buffer whose other entries name a page
-    of NaNs, so a read past a row or past the table shows."""
+    sequence's block-table row nor derail its neighbours: an oversized sequence computes exactly what it computes with
+    the length its row can address, a negative one what an empty one does (zeros), every other row is untouched, and
+    no unaddressed (NaN-filled) token is read.  Past a row lies the next sequence's row (other, valid pages: reading
+    them changes the result); past the last row lies the end of the table."""
     require_gfx950()
     page, width = 64, 4
-    lens_ok = [100, 0, width * page, 64, 200]
+    lens_ok = [100, 0, width * page, 64, width * page]
     case = _ragged_case(len(lens_ok), 32, 8, 128, page, lens_ok, torch.bfloat16, fp8=fp8, seed=23)
-    q, k, v, lens, table, ks, vs = case
-    assert table.shape[1] == width
-    nan_page = int(table[1, 0])                      # the spare page unused entries name: all NaN
-    big = torch.full((len(lens_ok) + 2, width + 3), nan_page, dtype=torch.int32)
-    big[1:-1, :width] = table
+    assert case[4].shape[1] == width
     dev = [None if t is None else t.to(DEV) for t in case]
-    dev[4] = big.to(DEV)[1:-1, :width]               # same values, row stride width + 3, NaN-page ids all around
-    op = PagedOp(len(lens_ok), 32, 8, k.shape[0], 128, page)
+    op = PagedOp(len(lens_ok), 32, 8, case[1].shape[0], 128, page)
     op.kernel_map = {kernel_key: op.kernel_map[kernel_key]}
     args = dev[:5] if not fp8 else dev
     want = op(*args).clone()
     torch.cuda.synchronize()
     assert torch.isfinite(want).all() and (want[1] == 0).all()
-    bad = torch.tensor([100, -7, 2 ** 31 - 1, 64, 200], dtype=torch.int32, device=DEV)
-    got = op(args[0], args[1], args[2], bad, *args[4:])
-    torch.cuda.synchronize()
-    assert torch.isfinite(got).all()
-    assert torch.equal(got, want)
-    bad2 = torch.tensor([100, -(2 ** 31), width * page + 1, 64, 200], dtype=torch.int32, device=DEV)
-    assert torch.equal(op(args[0], args[1], args[2], bad2, *args[4:]), want)
+    for bad in ([100, -7, 2 ** 31 - 1, 64, width * page + 1], [100, -(2 ** 31), width * page + 1, 64, 10 ** 9]):
+        got = op(args[0], args[1], args[2], torch.tensor(bad, dtype=torch.int32, device=DEV), *args[4:])
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all()
+        assert torch.equal(got, want)
 
 
 def _random_configs(n, seed):
