@@ -105,6 +105,24 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
                            int kernel, void* hip_stream);
 
 /*
+ * mi355_gqa_paged_decode() for callers that cannot allocate: the same call, with the library's own scratch in place of the
+ * workspace argument.  It has no counterpart in the reference (whose forward allocates glse / Output_partial with torch on
+ * every call, gqa_decode_paged.py:718-721); it is for callers that cannot call hipMalloc or hold a workspace -- code under
+ * HIP graph capture, tight serving loops, harnesses that forbid allocation.  It calls no hipMalloc / hipFree or other
+ * allocating routine; the scratch is an 80 MiB array in the library's device image, one per GPU, held until the process ends.
+ * Limits: calls whose workspace requirement (mi355_gqa_paged_decode_workspace) exceeds 80 MiB are refused with
+ * MI355_EWORKSPACE and a message (every plan of the MFMA kernel fits: at most 67.6 MB whatever the shape; the general
+ * kernel's plan grows with batch x splits and may not);
+ * all calls on one GPU share that GPU's array, so two calls that overlap in time on one GPU (different streams) race --
+ * keep such calls on one stream, or use mi355_gqa_paged_decode with separate workspaces.  Arguments as there.
+ */
+int mi355_gqa_paged_decode_static(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                  const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,
+                                  int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
+                                  int64_t n_phys_tokens, int q_dtype, int kv_dtype, float sm_scale, float softcap, int causal,
+                                  int num_split, int kernel, void* hip_stream);
+
+/*
  * GQA decode over a contiguous (un-paged) KV cache: one call = one forward of
  * GroupedQueryAttentionDecodeWithKVCacheFwdOp (src/tileops/ops/attention/gqa.py:1336-1350 ->
  * GQADecodeKernel.forward, src/tileops/kernels/attention/gqa_decode.py:555-612; custom-op argument lists

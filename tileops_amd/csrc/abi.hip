@@ -222,6 +222,33 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
   return MI355_OK;
 }
 
+// Scratch of the entry point that allocates nothing (mi355_gqa_paged_decode_static): one array per GPU, there from
+// the moment the code object is loaded until the process ends.  Host code never uses the array's name as an address:
+// the name is a host-side handle, the array's device address is asked for once per device and kept.
+constexpr size_t kStaticScratchBytes = (size_t)80 << 20;  // every plan of the MFMA kernel fits (at most 67.6 MB)
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+    (void)hipGetLastError();
+    return fail(MI355_EDEVICE, "no HIP device is current (these kernels need a gfx950 GPU)");
+  }
+  if (dev >= kMaxDevices) return fail(MI355_EUNSUPPORTED, "device index %d exceeds the %d devices the static scratch table holds", dev, kMaxDevices);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // this device's copy of the array (the current device's)
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return fail(MI355_ELAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return MI355_OK;
+}
+
 }  // namespace
 
 namespace mi355 {
@@ -282,6 +309,40 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
   return run_decode(q, k, v, k_scale, v_scale, seqlens, block_table, bt_row_stride, 0, 0, out, workspace, workspace_bytes,
                     batch, q_len, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype, kv_dtype, sm_scale, softcap,
                     causal, num_split, kernel, hip_stream);
+}
+
+int mi355_gqa_paged_decode_static(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+                                  const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out, int batch,
+                                  int q_len, int heads, int heads_kv, int dim, int page_size, int64_t n_phys_tokens, int q_dtype,
+                                  int kv_dtype, float sm_scale, float softcap, int causal, int num_split, int kernel,
+                                  void* hip_stream) {
+  int rc = check_shape(batch, q_len, heads, heads_kv, dim, page_size, q_dtype, kv_dtype);
+  if (rc) return rc;
+  if (batch == 0) return MI355_OK;
+  if (!q || !k || !v || !seqlens || !block_table || !out)
+    return fail(MI355_EINVAL, "q, k, v, seqlens, block_table and out must be non-null");
+  if (n_phys_tokens <= 0 || n_phys_tokens % page_size != 0)
+    return fail(MI355_EINVAL, "n_phys_tokens (%lld) must be a positive multiple of page_size (%d)", (long long)n_phys_tokens,
+                page_size);
+  if (bt_row_stride <= 0) return fail(MI355_EINVAL, "bt_row_stride must be positive");
+  if (kernel & kKernelFlagSkipCombine) return fail(MI355_EINVAL, "unknown kernel selector %d", kernel);
+  Plan plan;
+  rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan);
+  if (rc) return rc;
+  const size_t need = plan.part_o_bytes + plan.part_lse_bytes;
+  if (need > kStaticScratchBytes)
+    return fail(MI355_EWORKSPACE, "this call needs %zu bytes of scratch, the static buffer of mi355_gqa_paged_decode_static holds %zu: "
+                "use mi355_gqa_paged_decode with a workspace of the caller's", need, kStaticScratchBytes);
+  rc = check_device();
+  if (rc) return rc;
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  // Nothing in the scratch has to start at zero: the attention kernel writes every record and every partial slot that
+  // the merge reads in the same call, and the merge never touches a slot whose weight is zero.
+  return run_decode(q, k, v, k_scale, v_scale, seqlens, block_table, bt_row_stride, 0, 0, out, ws, kStaticScratchBytes, batch,
+                    q_len, heads, heads_kv, dim, page_size, n_phys_tokens, q_dtype, kv_dtype, sm_scale, softcap, causal, num_split,
+                    kernel, hip_stream);
 }
 
 // A contiguous cache is walked in 32-token tiles: the "page size" both kernels do their tile arithmetic with.

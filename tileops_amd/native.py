@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "mi355_last_error",
     "mi355_gqa_paged_decode_workspace",
     "mi355_gqa_paged_decode",
+    "mi355_gqa_paged_decode_static",
     "mi355_gqa_decode_workspace",
     "mi355_gqa_decode",
     "mi355_gqa_prefill_paged_workspace",
@@ -61,6 +62,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.mi355_gqa_paged_decode.restype = _c_int
     lib.mi355_gqa_paged_decode.argtypes = [
         _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_sz,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
+        _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
+    ]
+    lib.mi355_gqa_paged_decode_static.restype = _c_int
+    lib.mi355_gqa_paged_decode_static.argtypes = [
+        _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_int,
         _c_f32, _c_f32, _c_int, _c_int, _c_int, _c_vp,
     ]
@@ -210,6 +217,25 @@ def paged_decode(
         seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0), out.data_ptr(),
         workspace.data_ptr() if workspace is not None else None,
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        batch, q_len, heads, heads_kv, dim, page_size, k.shape[0],
+        dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
+        int(num_split), int(kernel), _stream_ptr(q.device)))
+
+
+def paged_decode_static(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
+    seqlens: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, *,
+    batch: int, q_len: int, heads: int, heads_kv: int, dim: int, page_size: int,
+    sm_scale: float, softcap: float, causal: bool, num_split: int = 0, kernel: int = KERNEL_AUTO,
+) -> None:
+    """The same call through the entry point that allocates nothing: the library's static scratch takes the place of the
+    workspace (calls needing more than 80 MiB are refused; calls overlapping on one GPU race)."""
+    lib = load()
+    _check(lib.mi355_gqa_paged_decode_static(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0), out.data_ptr(),
         batch, q_len, heads, heads_kv, dim, page_size, k.shape[0],
         dtype_code(q.dtype), dtype_code(k.dtype), float(sm_scale), float(softcap), int(bool(causal)),
         int(num_split), int(kernel), _stream_ptr(q.device)))
