@@ -240,7 +240,7 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // LDS ring: each fetches 1/SHW of every stage, and one barrier per tile makes all parts visible and retires the slot
 // that is refilled next.  All waves execute the same number of barriers because they own the same tile range.
 template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW, int D>
-__global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
+__global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT, D>;
   constexpr bool FP8 = G::FP8;
   constexpr int NJ = D / 32;    // 32-wide steps of the head dim in Q.K^T
@@ -675,7 +675,11 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
   // With an fp8 cache and several row blocks registers are short: V^T then stays in bytes until the PV product
   // consumes it (widened one 16-column block at a time, in between the MFMAs).
   constexpr bool LATE_V = FP8 && (NRB >= 2 || D == 256);
-  u32x4 va_op[LATE_V ? 1 : NDB];
+  // 16-bit cache, head dim 256, ring of eight (two waves per SIMD, 256 registers each): the V^T operands of a tile are
+  // 64 registers, as many as the K operands; V^T is read from LDS inside the value step, four 16-column blocks at a
+  // time, instead of being held across the softmax, and K in two halves of the head dim.
+  constexpr bool LATE_VREAD = !FP8 && D == 256 && SHW == 8;
+  u32x4 va_op[(LATE_V || LATE_VREAD) ? 1 : NDB];
   i32x2 vraw[LATE_V ? NDB : 1];
   u32x4 pk[NRB];
   float alpha[NRB];
@@ -686,16 +690,20 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
     f32x4 ksc[2], vsc[2];
     constexpr uint32_t HALF = 16 * G::ROW;  // bytes of one 16-token block of K (or V)
     if constexpr (!FP8) {
+      if constexpr (!LATE_VREAD) {
 #pragma unroll
-      for (int tb = 0; tb < 2; tb++)
+        for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
+          for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
+      }
+      if constexpr (!LATE_VREAD) {
 #pragma unroll
-      for (int db = 0; db < NDB; db++) {
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
-        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-        va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+        for (int db = 0; db < NDB; db++) {
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
+          u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+        }
       }
     } else {
       u32x4 kraw[2][NJ / 2];
@@ -747,6 +755,27 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
             for (int tb = 0; tb < 2; tb++)
               s_acc[tb][rb] = mma_fp8_k128(ka_op[tb][2 * h], ka_op[tb][2 * h + 1], qreg[rb][part * NCH + 2 * h],
                                            qreg[rb][part * NCH + 2 * h + 1], s_acc[tb][rb]);
+    } else if constexpr (LATE_VREAD) {
+      // the K operands in two halves of the head dim (32 registers each): read, multiply, read, multiply
+#pragma unroll
+      for (int hf = 0; hf < 2; hf++) {
+        u32x4 kh[2][NJ / 2];
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+          for (int jj = 0; jj < NJ / 2; jj++) {
+            const int j = hf * (NJ / 2) + jj;
+            kh[tb][jj] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jj = 0; jj < NJ / 2; jj++)
+#pragma unroll
+          for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++) s_acc[tb][rb] = Mma<QT>::run(kh[tb][jj], qreg[rb][hf * (NJ / 2) + jj], s_acc[tb][rb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < NJ; j++)
@@ -829,7 +858,33 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         __builtin_amdgcn_sched_barrier(0);  // one tile at a time: keeps the copies out of the accumulation registers short-lived
       }
   };
-  auto value_step = [&]() __attribute__((always_inline)) {
+  auto value_step = [&](const uint32_t SOFF) __attribute__((always_inline)) {
+    if constexpr (LATE_VREAD) {
+      constexpr uint32_t HALF = 16 * G::ROW;
+      constexpr int GB = 4;  // 16-column blocks per round of LDS reads
+      auto read_group = [&](int g0, u32x4* dst) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < GB; e++) {
+          const int db = g0 + e;
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
+          u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          dst[e] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+        }
+      };
+      u32x4 vt[2][GB];
+      read_group(0, vt[0]);
+#pragma unroll
+      for (int gi = 0; gi < NDB / GB; gi++) {
+        if (gi + 1 < NDB / GB) read_group((gi + 1) * GB, vt[(gi + 1) & 1]);  // the next round is in flight under this round's products
+#pragma unroll
+        for (int e = 0; e < GB; e++)
+#pragma unroll
+          for (int rb = 0; rb < NRB; rb++) o_acc[rb][gi * GB + e] = Mma<QT>::run(vt[gi & 1][e], pk[rb], o_acc[rb][gi * GB + e]);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the rounds apart: at most two rounds of operands are live
+      }
+      return;
+    }
 #pragma unroll
     for (int db = 0; db < NDB; db++) {
       u32x4 vt;
@@ -935,21 +990,21 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && D <= 128) ? 2 : 1) void paged_
         }
         if (LATE) issue_ahead(ring);
         moved = run_score_step(ring);
-        if constexpr ((SH && D <= 128) || (FP8 && NRB == 2)) {
+        if constexpr ((SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2)) {
           // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
           if (__builtin_expect(moved, 0)) rescale();
           moved = false;
         } else {
           if (__builtin_expect(moved, 0)) break;
         }
-        value_step();
+        value_step((uint32_t)ring * G::STAGE);
         ++u;
         ++cc.j;
         ring = ring + 1 == NS ? 0 : ring + 1;
       }
       if (moved) {  // rare after the first tiles of a sequence: finish this tile out of line, then re-enter
         rescale();
-        value_step();
+        value_step((uint32_t)ring * G::STAGE);
         ++u;
         ++cc.j;
         ring = ring + 1 == NS ? 0 : ring + 1;
@@ -1296,8 +1351,11 @@ int row_blocks_for(int rows, int dim) { return (rows <= 16 || dim == 256) ? 1 : 
 // fetch instructions per wave, one trip through the memory system per tile); an odd count is rounded up by one idle
 // row group.  Eight waves a compute unit either way (accumulators of two row blocks fit ordinary vector registers);
 // the ring takes the LDS that leaves (a 16-bit stage is 16 KiB, an fp8 one 8.25 KiB).
-// (128-byte rows, fp8 or head dim 64, have four fetch instructions per K tile, 64-byte rows two; 512-byte rows, head
-// dim 256, keep their accumulators in AGPRs and run one wave per SIMD)
+// (128-byte rows, fp8 or head dim 64, have four fetch instructions per K tile, 64-byte rows two.  Head dim 256 has one
+// row block per wave: unshared waves and rings of two or four keep their accumulators in AGPRs and run one wave per
+// SIMD; a ring of eight reads its K and V^T operands from LDS in portions -- K in two halves of the head dim, V^T four
+// 16-column blocks at a time inside the value step -- so that a wave fits 256 registers and two run per SIMD: 128
+// query rows per trip of a K/V tile through the memory system instead of 64, half the fetch instructions per wave.)
 int ring_waves_for(int rows, int nrb, int max_ring) {
   const int n = row_groups(rows, nrb);
   if (n <= 1) return 1;
@@ -1307,16 +1365,16 @@ int ring_waves_for(int rows, int nrb, int max_ring) {
   return 2;
 }
 // Largest ring for a row width: a ring splits the fetch instructions of a K tile (one per KiB: 8, 4 or 2 for rows of
-// 256, 128 or 64 bytes) evenly over its waves; head dim 256 stops at four waves, one per SIMD.
+// 256, 128 or 64 bytes; 16 for the 512-byte rows of a 16-bit cache at head dim 256) evenly over its waves.
 int max_ring_for(int dim, bool fp8) {
   const int row = dim * (fp8 ? 1 : 2);
-  return (row == 256 && dim != 256) ? 8 : (row == 64 ? 2 : 4);
+  return (row == 256 || row == 512) ? 8 : (row == 64 ? 2 : 4);
 }
 
 template <typename QT, typename KVT, int D>
 const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, hipStream_t s) {
   constexpr bool SMALL = Geom<KVT, D>::ROW <= 128;  // 8 KiB stages or less: eight unshared waves a CU, four-deep pair rings
-  constexpr bool WIDE = Geom<KVT, D>::ROW == 512;   // 32 KiB stages, accumulators in AGPRs: one wave per SIMD at most
+  constexpr bool WIDE = Geom<KVT, D>::ROW == 512;   // 32 KiB stages: two unshared waves per workgroup
   constexpr int NWU = SMALL ? 8 : (WIDE ? 2 : 4);   // unshared waves per workgroup (two stages each fill the LDS)
   if (p.rows <= 16) return launch_t4<QT, KVT, 1, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
   constexpr int NRB = D == 256 ? 1 : 2;  // == row_blocks_for(rows > 16, D)
@@ -1327,7 +1385,7 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
       if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of four waves for this row width";
     default:
-      if constexpr (!SMALL && D != 256) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
@@ -1353,7 +1411,7 @@ int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
   const int n_rg = ring_row_groups(rows, nrb, shw);
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
-  const int waves_per_cu = dim == 256 ? ((shw > 1 || fp8) ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
+  const int waves_per_cu = dim == 256 ? (shw == 8 ? 8 : (shw > 1 || fp8) ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
   const int64_t waves = (int64_t)device_cu_count() * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
