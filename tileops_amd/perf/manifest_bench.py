@@ -20,7 +20,6 @@ from __future__ import annotations
 
 import argparse
 import statistics
-import subprocess
 import sys
 import xml.etree.ElementTree as ET
 from datetime import datetime
@@ -62,10 +61,11 @@ class BenchmarkReport:
             lines.append(f"- **GPU model**: {props.name} ({getattr(props, 'gcnArchName', '?')}, {props.multi_processor_count} CUs)")
         else:
             lines.append("- **GPU model**: N/A (no device)")
+        # The amdgpu kernel module publishes its version in sysfs; no child process is started from a process that
+        # holds the GPU.
         try:
-            out = subprocess.run(["rocm-smi", "--showdriverversion"], capture_output=True, text=True, timeout=10).stdout
-            driver = next((ln.split(":")[-1].strip() for ln in out.splitlines() if "Driver version" in ln), "N/A")
-        except (FileNotFoundError, subprocess.TimeoutExpired):
+            driver = Path("/sys/module/amdgpu/version").read_text().strip() or "N/A"
+        except OSError:
             driver = "N/A"
         lines.append(f"- **Driver version**: {driver}")
         return lines
