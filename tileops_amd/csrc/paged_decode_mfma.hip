@@ -196,7 +196,7 @@ struct Cursor {
 __device__ __forceinline__ void cursor_load_lens(Cursor& c, const DecodeParams& p, int base) {
   const int lane = threadIdx.x & 63;
   c.lens_base = base;
-  c.lens = seq_len_of(p, min(base + lane, p.batch - 1));
+  c.lens = seq_len_of<true>(p, min(base + lane, p.batch - 1));
   // Land the load here.  Left to itself the compiler waits for it where the register is next read -- after the
   // join with the path that did not load, i.e. on every pass -- and its wait (vmcnt 0) also drains every
   // direct-to-LDS load in flight.  An empty asm that reads the register moves the wait into this rare block.
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   int T = 0;
   for (int base = 0; base < p.batch; base += 64) {
     int b = base + lane;
-    int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
+    int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
 #pragma unroll
     for (int m = 1; m < 64; m <<= 1) n += __shfl_xor(n, m, 64);
     T += n;
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     int carry = 0;
     for (int base = 0; base < p.batch; base += 64) {
       int b = base + lane;
-      int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
+      int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
       int incl = n;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     int carry = 0, b0 = -1, pre0 = 0;
     for (int base = 0; base < p.batch && b0 < 0; base += 64) {
       int b = base + lane;
-      int n = b < p.batch ? units_of(seq_len_of(p, b)) : 0;
+      int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
       int incl = n;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
