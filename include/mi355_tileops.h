@@ -235,6 +235,21 @@ int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int3
                         const int32_t* block_table, int64_t bt_row_stride, int batch, int heads_kv, int dim,
                         int page_size, int64_t n_phys_tokens, int x_dtype, void* hip_stream);
 
+/*
+ * The facts behind the value checks that the reference's paged prefill op makes on the host before it launches
+ * (GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp._validate_forward_inputs, src/tileops/ops/attention/gqa.py:997-1040:
+ * each there a device-to-host read of its own), reduced by one small kernel into ten int32 in device memory so that a
+ * caller reads them in one transfer:
+ *   facts[0], facts[1]  k_scale[0], v_scale[0] finite and positive (1/0; a null scale pointer counts as good)
+ *   facts[2] cu_seqlens_q[0]           facts[3] min q_len     facts[4] cu_seqlens_q[batch]   facts[5] max q_len
+ *   facts[6] min cache_seqlens         facts[7] max (cache_seqlens + q_len), saturated to int32
+ *   facts[8], facts[9]  min and max block_table entry over the batch x max_pages_per_req entries
+ * Nothing is judged here: which values are errors, and their messages, stay with the caller.
+ */
+int mi355_prefill_input_facts(const int32_t* cu_seqlens_q, const int32_t* cache_seqlens, const int32_t* block_table,
+                              int64_t bt_row_stride, const float* k_scale, const float* v_scale, int batch,
+                              int max_pages_per_req, int32_t* facts, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

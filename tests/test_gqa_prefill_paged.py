@@ -300,6 +300,56 @@ def test_validate_inputs_false_skips_the_device_reads_and_nothing_else():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fp8", [False, True])
+def test_value_checks_cost_one_host_read(fp8):
+    """The reference's value checks (scales, cu_seqlens_q, cache_seqlens, capacity, block-table range) are reduced on
+    the device and cross to the host in one transfer: torch's sync debug mode reports one synchronising call."""
+    import warnings
+    require_gfx950()
+    case = [t.to(DEV) for t in _case([33, 48], [67, 80], 8, 2, 64, torch.float16, fp8=fp8)]
+    op = PrefillOp(batch=2, heads=8, heads_kv=2, max_pages_per_req=8, page_size=64, dim=64, cache_dtype=FP8 if fp8 else None)
+    op(*[t.clone() for t in case], 48)  # builds the kernel object and its tables
+    torch.cuda.synchronize()
+    before = torch.cuda.get_sync_debug_mode()
+    torch.cuda.set_sync_debug_mode("warn")
+    try:
+        with warnings.catch_warnings(record=True) as seen:
+            warnings.simplefilter("always")
+            op._validate_forward_inputs(*case, 48)
+    finally:
+        torch.cuda.set_sync_debug_mode(before)
+    syncs = [w for w in seen if "synchroniz" in str(w.message).lower()]
+    assert len(syncs) == 1, [str(w.message) for w in seen]
+
+
+@pytest.mark.gpu
+def test_input_facts_entry_point_against_torch():
+    """mi355_prefill_input_facts on a strided block table with negative entries, a length sum that leaves int32 and a
+    bad scale, against the same reductions in torch."""
+    require_gfx950()
+    g = torch.Generator().manual_seed(5)
+    batch, width = 37, 300
+    q_lens = torch.randint(-3, 900, (batch,), generator=g, dtype=torch.int32)
+    cu = torch.full((batch + 1,), 7, dtype=torch.int32)
+    cu[1:] += torch.cumsum(q_lens, 0).to(torch.int32)
+    cache = torch.randint(-5, 1 << 20, (batch,), generator=g, dtype=torch.int32)
+    cache[3] = 2**31 - 5  # with any positive q_len the sum leaves int32: the fact saturates
+    q_lens[3] = 11
+    cu[4:] += 11 - (cu[4] - cu[3])
+    wide = torch.randint(-9, 1 << 22, (batch, 512), generator=g, dtype=torch.int32)
+    table_dev = wide.to(DEV)[:, :width]  # rows 512 entries apart, 300 of them addressed
+    assert not table_dev.is_contiguous()
+    ks, vs = torch.tensor([0.5], device=DEV), torch.tensor([float("nan")], device=DEV)
+    got = native.prefill_input_facts(cu.to(DEV), cache.to(DEV), table_dev, ks, vs)
+    ql = (cu[1:] - cu[:-1]).to(torch.int64)
+    tot = torch.clamp(cache.to(torch.int64) + ql, -2**31, 2**31 - 1)
+    table = wide[:, :width]
+    want = [1, 0, int(cu[0]), int(ql.min()), int(cu[-1]), int(ql.max()), int(cache.min()), int(tot.max()), int(table.min()), int(table.max())]
+    assert got == want and want[7] == 2**31 - 1
+    assert native.prefill_input_facts(cu.to(DEV), cache.to(DEV), table_dev, None, None)[:2] == [1, 1]
+
+
+@pytest.mark.gpu
 def test_prefill_rejects_bad_calls():
     require_gfx950()
     case = [t.to(DEV) for t in _case([4, 4], [10, 10], 8, 2, 64, torch.float16)]
@@ -317,6 +367,23 @@ def test_prefill_rejects_bad_calls():
     bad = list(case)
     bad[3] = case[3].to(torch.bfloat16)
     with pytest.raises(ValueError, match="Expected k_pages.dtype"):
+        op(*bad, 4)
+    bad = list(case)
+    bad[8] = torch.tensor([-1, 10], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="cache_seqlens must be non-negative"):
+        op(*bad, 4)
+    bad = list(case)
+    bad[7] = torch.tensor([0, 6, 4], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="cu_seqlens_q must be non-decreasing"):
+        op(*bad, 6)
+    bad = list(case)
+    bad[7] = torch.tensor([0, 4, 7], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match=r"cu_seqlens_q\[-1\] .7. must equal q.shape\[0\] .8."):
+        op(*bad, 4)
+    bad = list(case)
+    bad[9] = case[9].clone()
+    bad[9][1, 3] = -2
+    with pytest.raises(ValueError, match="non-negative physical page ids"):
         op(*bad, 4)
 
 

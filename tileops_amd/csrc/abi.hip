@@ -599,4 +599,17 @@ int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int3
   return MI355_OK;
 }
 
+int mi355_prefill_input_facts(const int32_t* cu_seqlens_q, const int32_t* cache_seqlens, const int32_t* block_table,
+                              int64_t bt_row_stride, const float* k_scale, const float* v_scale, int batch, int max_pages_per_req,
+                              int32_t* facts, void* hip_stream) {
+  if (batch <= 0 || max_pages_per_req <= 0) return fail(MI355_EINVAL, "batch and max_pages_per_req must be positive");
+  if (bt_row_stride < max_pages_per_req) return fail(MI355_EINVAL, "bt_row_stride must be at least max_pages_per_req");
+  if (!cu_seqlens_q || !cache_seqlens || !block_table || !facts) return fail(MI355_EINVAL, "null pointer argument");
+  if (int rc = check_device()) return rc;
+  const char* err = launch_prefill_input_facts(cu_seqlens_q, cache_seqlens, block_table, bt_row_stride, k_scale, v_scale, batch,
+                                               max_pages_per_req, facts, (hipStream_t)hip_stream);
+  if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+  return MI355_OK;
+}
+
 }  // extern "C"

@@ -128,6 +128,9 @@ const char* launch_rope_append_chunk(const void* q, const void* k_new, const voi
                                      int page_size, int64_t n_pages, int x_dtype, hipStream_t s);
 const char* launch_merge_two(const float* o_a, const float* lse_a, const float* o_b, const float* lse_b, void* out,
                              int64_t rows, int dim, int q_dtype, hipStream_t s);
+const char* launch_prefill_input_facts(const int32_t* cu_q, const int32_t* cache_seqlens, const int32_t* block_table,
+                                       int64_t bt_row_stride, const float* k_scale, const float* v_scale, int batch, int max_pages,
+                                       int32_t* facts, hipStream_t s);
 const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, const int32_t* seqlens,
                                  const int32_t* block_table, int64_t bt_row_stride, int batch, int heads_kv, int dim,
                                  int page_size, int64_t n_pages, int x_dtype, hipStream_t s);

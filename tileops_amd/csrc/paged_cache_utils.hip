@@ -1,4 +1,5 @@
 // Page-table utilities for gfx950: the index-probe gather and the FP8 KV-cache append.
+#include <climits>
 #include "common.h"
 #include "device_utils.h"
 
@@ -88,6 +89,72 @@ const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, c
   else
     hipLaunchKernelGGL(kv_append_fp8_kernel<fp16_tag>, grid, dim3(64), 0, s, (const uint16_t*)x_new, (uint8_t*)cache, scale,
                        seqlens, block_table, bt_row_stride, heads_kv, dim, page_size, n_pages);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
+// The facts behind the value checks of the reference's paged prefill op (src/tileops/ops/attention/gqa.py:997-1040),
+// reduced on the device so that the host reads them in one transfer instead of one per check:
+//   facts[0] k_scale finite and positive (1/0)      facts[1] v_scale finite and positive (1/0)
+//   facts[2] cu_q[0]                                 facts[3] min over b of cu_q[b+1] - cu_q[b]
+//   facts[4] cu_q[batch]                             facts[5] max over b of cu_q[b+1] - cu_q[b]
+//   facts[6] min cache_seqlens                       facts[7] max over b of cache_seqlens[b] + q_len[b]   (64-bit sums, saturated)
+//   facts[8] min block_table entry                   facts[9] max block_table entry
+// One workgroup of 256 threads; the block table (batch x max_pages entries, rows bt_row_stride apart) is the long loop.
+__global__ __launch_bounds__(256) void prefill_input_facts_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
+                                                                  const int32_t* __restrict__ block_table, int64_t bt_row_stride,
+                                                                  const float* __restrict__ k_scale, const float* __restrict__ v_scale,
+                                                                  int batch, int max_pages, int32_t* __restrict__ facts) {
+  __shared__ int red[6][256];
+  const int t = threadIdx.x;
+  int min_q = INT_MAX, max_q = INT_MIN, min_c = INT_MAX, max_tot = INT_MIN, min_p = INT_MAX, max_p = INT_MIN;
+  for (int b = t; b < batch; b += 256) {
+    const int ql = cu_q[b + 1] - cu_q[b], c = cache_seqlens[b];
+    const int64_t tot = (int64_t)c + ql;
+    min_q = min(min_q, ql);
+    max_q = max(max_q, ql);
+    min_c = min(min_c, c);
+    max_tot = max(max_tot, (int)min(max(tot, (int64_t)INT_MIN), (int64_t)INT_MAX));
+  }
+  const int64_t n_entries = (int64_t)batch * max_pages;
+  for (int64_t i = t; i < n_entries; i += 256) {
+    const int v = block_table[(i / max_pages) * bt_row_stride + i % max_pages];
+    min_p = min(min_p, v);
+    max_p = max(max_p, v);
+  }
+  red[0][t] = min_q; red[1][t] = max_q; red[2][t] = min_c; red[3][t] = max_tot; red[4][t] = min_p; red[5][t] = max_p;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) {
+      red[0][t] = min(red[0][t], red[0][t + w]);
+      red[1][t] = max(red[1][t], red[1][t + w]);
+      red[2][t] = min(red[2][t], red[2][t + w]);
+      red[3][t] = max(red[3][t], red[3][t + w]);
+      red[4][t] = min(red[4][t], red[4][t + w]);
+      red[5][t] = max(red[5][t], red[5][t + w]);
+    }
+    __syncthreads();
+  }
+  if (t == 0) {
+    const float ks = k_scale ? k_scale[0] : 1.f, vs = v_scale ? v_scale[0] : 1.f;
+    facts[0] = (isfinite(ks) && ks > 0.f) ? 1 : 0;
+    facts[1] = (isfinite(vs) && vs > 0.f) ? 1 : 0;
+    facts[2] = cu_q[0];
+    facts[3] = red[0][0];
+    facts[4] = cu_q[batch];
+    facts[5] = red[1][0];
+    facts[6] = red[2][0];
+    facts[7] = red[3][0];
+    facts[8] = red[4][0];
+    facts[9] = red[5][0];
+  }
+}
+
+const char* launch_prefill_input_facts(const int32_t* cu_q, const int32_t* cache_seqlens, const int32_t* block_table,
+                                       int64_t bt_row_stride, const float* k_scale, const float* v_scale, int batch, int max_pages,
+                                       int32_t* facts, hipStream_t s) {
+  hipLaunchKernelGGL(prefill_input_facts_kernel, dim3(1), dim3(256), 0, s, cu_q, cache_seqlens, block_table, bt_row_stride, k_scale,
+                     v_scale, batch, max_pages, facts);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }

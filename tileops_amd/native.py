@@ -36,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "mi355_gqa_prefill_paged_rope",
     "mi355_gather_probe",
     "mi355_kv_append_fp8",
+    "mi355_prefill_input_facts",
 )
 
 
@@ -104,6 +105,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     ]
     lib.mi355_gather_probe.restype = _c_int
     lib.mi355_gather_probe.argtypes = [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_int, _c_i64, _c_i64, _c_int, _c_i64, _c_vp]
+    lib.mi355_prefill_input_facts.restype = _c_int
+    lib.mi355_prefill_input_facts.argtypes = [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_int, _c_int, _c_vp, _c_vp]
     lib.mi355_kv_append_fp8.restype = _c_int
     lib.mi355_kv_append_fp8.argtypes = [
         _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_int, _c_vp,
@@ -352,3 +355,17 @@ def kv_append_fp8(x_new: torch.Tensor, cache: torch.Tensor, scale: torch.Tensor,
         x_new.data_ptr(), cache.data_ptr(), scale.data_ptr(), seqlens.data_ptr(), block_table.data_ptr(),
         block_table.stride(0), batch, heads_kv, dim, page_size, cache.shape[0], dtype_code(x_new.dtype),
         _stream_ptr(cache.device)))
+
+
+def prefill_input_facts(cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor, block_table: torch.Tensor,
+                        k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor]) -> list[int]:
+    """The ten facts behind the paged prefill op's value checks (see ``mi355_prefill_input_facts``): one small kernel,
+    one transfer to the host."""
+    require_gfx950(block_table.device)
+    lib = load()
+    facts = torch.empty(10, dtype=torch.int32, device=block_table.device)
+    _check(lib.mi355_prefill_input_facts(
+        cu_seqlens_q.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        k_scale.data_ptr() if k_scale is not None else None, v_scale.data_ptr() if v_scale is not None else None,
+        cache_seqlens.shape[0], block_table.shape[1], facts.data_ptr(), _stream_ptr(block_table.device)))
+    return facts.tolist()

@@ -23,6 +23,7 @@ from typing import Dict, Optional
 
 import torch
 
+from . import native
 from .backend import Target
 from .kernels import (
     DECODE_KEYS, PAGED_DECODE_KEYS, PAGED_PREFILL_KEYS, AttentionCall, GQADecodeKernel, GQADecodeMfmaKernel,
@@ -547,29 +548,31 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
         for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
             if t.dtype != torch.float32:
                 raise ValueError(f"{name} must have dtype torch.float32, got {t.dtype}")
-            if self.validate_inputs and cache_dtype == FP8 and not torch.all(torch.isfinite(t) & (t > 0)).item():
-                raise ValueError(f"{name} must contain finite positive values")
         for name, t in (("cu_seqlens_q", cu_seqlens_q), ("cache_seqlens", cache_seqlens), ("block_table", block_table)):
             if t.dtype != torch.int32:
                 raise ValueError(f"{name} must have dtype torch.int32, got {t.dtype}")
         if not self.validate_inputs:
             return
-        cu = cu_seqlens_q.cpu()
-        if int(cu[0]) != 0:
+        # The value checks of the reference (gqa.py:997-1040), in its order and with its messages.  The reference reads
+        # each fact from the device on its own (five to seven round trips with the GPU idle in between); here the facts
+        # are reduced by one small kernel of the library into ten integers that cross to the host once.
+        facts = native.prefill_input_facts(cu_seqlens_q, cache_seqlens, block_table, k_scale if cache_dtype == FP8 else None,
+                                           v_scale if cache_dtype == FP8 else None)
+        for name, ok in zip(("k_scale", "v_scale"), facts[:2]):
+            if not ok:
+                raise ValueError(f"{name} must contain finite positive values")
+        facts = facts[2:]
+        cu_first, min_q, total_q, actual_max_q, min_cache, max_total_len, min_page, max_page = (int(x) for x in facts)
+        if cu_first != 0:
             raise ValueError("cu_seqlens_q[0] must be 0")
-        q_lens = cu[1:] - cu[:-1]
-        if bool((q_lens < 0).any()):
+        if min_q < 0:
             raise ValueError("cu_seqlens_q must be non-decreasing")
-        total_q = int(cu[-1])
         if total_q != q.shape[0]:
             raise ValueError(f"cu_seqlens_q[-1] ({total_q}) must equal q.shape[0] ({q.shape[0]})")
-        actual_max_q = int(q_lens.max())
         if max_seqlen_q < actual_max_q:
             raise ValueError(f"max_seqlen_q ({max_seqlen_q}) must be >= actual max Q sequence length ({actual_max_q})")
-        cache = cache_seqlens.cpu()
-        if int(cache.min()) < 0:
+        if min_cache < 0:
             raise ValueError("cache_seqlens must be non-negative")
-        max_total_len = int((cache + q_lens).max())
         if max_total_len > self.max_cache_len:
             raise ValueError("cache_seqlens + q_len exceeds paged KV capacity: "
                              f"max total length {max_total_len}, capacity {self.max_cache_len}")
@@ -577,7 +580,6 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
             raise ValueError("cache_seqlens + q_len exceeds RoPE max_position: "
                              f"max total length {max_total_len}, max_position {self.max_position}")
         num_pages = k_pages.shape[0] // self.page_size
-        min_page, max_page = int(block_table.min().item()), int(block_table.max().item())
         if min_page < 0:
             raise ValueError("block_table must contain non-negative physical page ids")
         if max_page >= num_pages:
