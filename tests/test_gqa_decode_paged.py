@@ -461,6 +461,29 @@ def test_kv_append_fp8_matches_the_quantizer_bit_for_bit():
     assert torch.equal(sd.cpu()[~touched], before_s.cpu()[~touched])
 
 
+def test_kv_append_fp8_writes_nothing_for_positions_the_block_table_row_does_not_address():
+    """Lengths of 0 (position -1) and beyond the row's pages: the append skips them instead of reading a page id from
+    the next row (or past the table) and writing into another sequence's page."""
+    require_gfx950()
+    page, H_kv, D, B, width = 64, 8, 128, 4, 3
+    lens = [0, width * page + 1, 70, width * page + 500]  # the last row's overrun would leave the table
+    case = _ragged_case(B, 32, H_kv, D, page, [1, 1, 130, 1], torch.bfloat16, fp8=True, seed=35, poison=False)  # table of three pages a row
+    q, k8, v8, _, table, ks, vs = case
+    assert table.shape == (B, width) and table.is_contiguous()
+    x_new = torch.randn(B, H_kv, D, generator=torch.Generator().manual_seed(36)).to(torch.bfloat16)
+    want_q, want_s = quantize_kv_per_token(x_new)
+    kd, sd = k8.to(DEV), ks.to(DEV)
+    before_k, before_s = kd.clone(), sd.clone()
+    native.kv_append_fp8(x_new.to(DEV), kd, sd, torch.tensor(lens, dtype=torch.int32, device=DEV), table.to(DEV), page)
+    torch.cuda.synchronize()
+    phys = int(table[2, 69 // page]) * page + 69 % page
+    touched = torch.zeros(k8.shape[0], dtype=torch.bool)
+    touched[phys] = True
+    assert torch.equal(kd[phys].cpu().view(torch.uint8), want_q[2].view(torch.uint8)) and torch.equal(sd[phys].cpu(), want_s[2])
+    assert torch.equal(kd.cpu().view(torch.uint8)[~touched], before_k.cpu().view(torch.uint8)[~touched])
+    assert torch.equal(sd.cpu()[~touched], before_s.cpu()[~touched])
+
+
 def test_external_builder_path_runs_the_same_kernels():
     """The plug-in's build_kernel, reached through the seam, gives the same bits as the in-tree path."""
     require_gfx950()

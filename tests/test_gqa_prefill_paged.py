@@ -323,6 +323,41 @@ def test_value_checks_cost_one_host_read(fp8):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["plain", "fp8", "rope"])
+def test_chunk_tokens_past_the_block_table_row_are_not_appended(mode):
+    """With the value checks off, a chunk that overruns its sequence's pages (cache 120 + 20 new tokens on two 64-token
+    pages) appends the eight tokens that fit and drops the rest: the pool afterwards differs from the pool before in
+    exactly the rows the table addresses, and no other sequence's pages are written."""
+    require_gfx950()
+    page, max_pages, heads, heads_kv, dim, dtype = 64, 2, 8, 2, 64, torch.float16
+    q_lens, old_lens = [20, 5], [120, 10]
+    fp8, rope = mode == "fp8", mode == "rope"
+    case = _case(q_lens, old_lens, heads, heads_kv, dim, dtype, fp8=fp8, page=page, max_pages=max_pages, seed=21)
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+    op = PrefillOp(batch=2, heads=heads, heads_kv=heads_kv, max_pages_per_req=max_pages, page_size=page, dim=dim,
+                   cache_dtype=FP8 if fp8 else None, fuse_rope=rope, max_position=256 if rope else None, validate_inputs=False)
+    dev = [t.to(DEV) for t in case]
+    out = op(*dev, max(q_lens))
+    torch.cuda.synchronize()
+    assert out.shape == q.shape
+    written = torch.zeros(k_pages.shape[0], dtype=torch.bool)
+    for b, (n, old) in enumerate(zip(q_lens, old_lens)):
+        for i in range(n):
+            t = old + i
+            if t >= max_pages * page:
+                continue
+            pos = physical_pos(table, b, t, page)
+            written[pos] = True
+            if not rope:  # values are copied (or quantised) as they are; rotated keys are checked by the rope tests
+                want_v = quantize_per_tensor(v_new[int(cu[b]) + i], vs) if fp8 else v_new[int(cu[b]) + i]
+                assert torch.equal(dev[4][pos].cpu().view(torch.uint8), want_v.view(torch.uint8))
+    assert int(written.sum()) == 8 + 5
+    for after, before in ((dev[3], k_pages), (dev[4], v_pages)):
+        assert torch.equal(after.cpu().view(torch.uint8)[~written], before.view(torch.uint8)[~written])
+        assert not torch.equal(after.cpu().view(torch.uint8)[written], before.view(torch.uint8)[written])
+
+
+@pytest.mark.gpu
 def test_input_facts_entry_point_against_torch():
     """mi355_prefill_input_facts on a strided block table with negative entries, a length sum that leaves int32 and a
     bad scale, against the same reductions in torch."""
