@@ -46,6 +46,30 @@ def _config(name: str):
     return config_from_workload(row, name, DESCRIPTIONS[name]), op_name, label
 
 
+def _device_busy_ms(fn, flush, calls: int):
+    """Mean over ``calls`` flushed calls of the summed durations of this library's kernels in one call, from the torch
+    profiler's device events; None when the profiler delivers none."""
+    try:
+        import torch
+        from torch.profiler import ProfilerActivity, profile
+
+        totals = []
+        for i in range(calls):
+            flush(i)
+            torch.cuda.synchronize()
+            with profile(activities=[ProfilerActivity.CUDA]) as prof:
+                fn()
+                torch.cuda.synchronize()
+            evs = [e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA and "mi355" in e.name]
+            if not evs:
+                return None
+            totals.append(sum(e.device_time for e in evs) / 1e3)
+        return sum(totals) / len(totals)
+    except Exception as exc:  # noqa: BLE001 - optional evidence; the timed figures above do not depend on it
+        print(f"device-busy time not measured: {exc!r}", file=sys.stderr)
+        return None
+
+
 def _timed_steps(fn, flush, steps: int) -> tuple[list[float], float]:
     """``steps`` calls, each after a cache flush and between its own pair of events on the stream the kernels run on."""
     import torch
@@ -135,6 +159,11 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         graph_ms, graph_median_ms = sum(g_ms) / steps, statistics.median(g_ms)
         torch.cuda.synchronize()
 
+    # Device-busy time of a whole call: the sum of the durations of the kernels it launches (attention + merge), launch
+    # latency and gaps excluded -- the quantity the reference's own timing protocol reports (its benchmarks take the
+    # per-iteration device-busy time from the profiler, benchmarks/timing.py:527-585).  Ten flushed calls.
+    busy_ms = _device_busy_ms(lambda: op(*args), flush, 10)
+
     op.observe_call(inp.real_seqlen_kv, cfg.kv_dtype)
     flops, total_bytes = op.eval_roofline()
     lens = inp.real_seqlen_kv.cpu().to(torch.int64)
@@ -181,6 +210,8 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
                      "traffic": traffic, "traffic_source": f"{TRAFFIC_SOURCE} (rocprofv3 FETCH_SIZE/WRITE_SIZE of an earlier profiler run, not counted in this run)"},
         "wall_s_timed_region": wall,
     }
+    if busy_ms is not None:
+        res["whole_call"].update({"us_device_busy_mean": busy_ms * 1e3, "kv_read_frac_of_peak_device_busy": gbs(kv_read, busy_ms) / HBM_PEAK_GBS})
     if graph_ms is not None:
         res["whole_call"].update({
             "us_graph_mean": graph_ms * 1e3, "us_graph_median": graph_median_ms * 1e3,
