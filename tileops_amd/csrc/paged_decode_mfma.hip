@@ -679,28 +679,46 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   // 64 registers, as many as the K operands; V^T is read from LDS inside the value step, four 16-column blocks at a
   // time, instead of being held across the softmax, and K in two halves of the head dim.
   constexpr bool LATE_VREAD = !FP8 && D == 256 && SHW == 8;
+  // The same ring with an FP8 cache: the 32 registers of V^T bytes are read inside the value step as well, four 16-column
+  // blocks at a time, and widened there.
+  constexpr bool LATE_VREAD8 = FP8 && D == 256 && SHW == 8;
   u32x4 va_op[(LATE_V || LATE_VREAD) ? 1 : NDB];
-  i32x2 vraw[LATE_V ? NDB : 1];
+  i32x2 vraw[(LATE_V && !LATE_VREAD8) ? NDB : 1];
   u32x4 pk[NRB];
   float alpha[NRB];
+  // LDS address of a read in ring slot offset SOFF.  Where SOFF is a run-time value (two row blocks: one copy of the tile
+  // body for all slots) the slot is added to each distinct lane base once and pinned there, so that the reads of a base
+  // differ by immediates only; left to itself the compiler forms (SOFF + constant) per read and spends one vector add on
+  // every one of them (24 a tile for a 16-bit cache).  With a constant SOFF everything folds into the immediate anyway.
+  auto in_slot = [&](uint32_t base, const uint32_t SOFF) __attribute__((always_inline)) -> uint32_t {
+    uint32_t a = base + SOFF;
+    if constexpr (NRB != 1 || LATE_VREAD) asm volatile("" : "+v"(a));
+    return a;
+  };
   auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
     u32x4 ka_op[2][NJ];
     f32x4 ksc[2], vsc[2];
     constexpr uint32_t HALF = 16 * G::ROW;  // bytes of one 16-token block of K (or V)
+    uint32_t kb[NKA];
+#pragma unroll
+    for (int i = 0; i < NKA; i++) kb[i] = in_slot(kaddr[i], SOFF);
     if constexpr (!FP8) {
       if constexpr (!LATE_VREAD) {
 #pragma unroll
         for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-          for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
+          for (int j = 0; j < NJ; j++) ka_op[tb][j] = *LDS_AT(u32x4, kb[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
       }
       if constexpr (!LATE_VREAD) {
+        uint32_t vb[NDB < 8 ? NDB : 8];
+#pragma unroll
+        for (int i = 0; i < (NDB < 8 ? NDB : 8); i++) vb[i] = in_slot(vaddr[i], SOFF);
 #pragma unroll
         for (int db = 0; db < NDB; db++) {
-          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
-          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vb[db & 7] + ((db >> 3) * 256)));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vb[db & 7] + (HALF + (db >> 3) * 256)));
           u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
           va_op[db] = u32x4{l2[0], l2[1], h2[0], h2[1]};
         }
@@ -711,14 +729,17 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-        for (int jj = 0; jj < NJ / 2; jj++) kraw[tb][jj] = *LDS_AT(u32x4, kaddr[jj] + (SOFF + tb * HALF));
+        for (int jj = 0; jj < NJ / 2; jj++) kraw[tb][jj] = *LDS_AT(u32x4, kb[jj] + (tb * HALF));
+      const uint32_t sb = in_slot(saddr, SOFF);
 #pragma unroll
       for (int tb = 0; tb < 2; tb++) {
-        ksc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 64 * tb));
-        vsc[tb] = *LDS_AT(f32x4, saddr + (SOFF + 128 + 64 * tb));
+        ksc[tb] = *LDS_AT(f32x4, sb + (64 * tb));
+        vsc[tb] = *LDS_AT(f32x4, sb + (128 + 64 * tb));
       }
+      if constexpr (!LATE_VREAD8) {
 #pragma unroll
-      for (int db = 0; db < NDB; db++) vnow[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[db] + SOFF));
+        for (int db = 0; db < NDB; db++) vnow[db] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, in_slot(vaddr[db], SOFF)));
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int tb = 0; tb < 2; tb++)
@@ -731,10 +752,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
             ka_op[tb][2 * jj + 1] = widen8<QT>(kraw[tb][jj][2], kraw[tb][jj][3]);
           }
         }
+      if constexpr (!LATE_VREAD8) {
 #pragma unroll
-      for (int db = 0; db < NDB; db++) {
-        if constexpr (LATE_V) vraw[db] = vnow[db];
-        else va_op[db] = widen8<QT>((uint32_t)vnow[db][0], (uint32_t)vnow[db][1]);
+        for (int db = 0; db < NDB; db++) {
+          if constexpr (LATE_V) vraw[db] = vnow[db];
+          else va_op[db] = widen8<QT>((uint32_t)vnow[db][0], (uint32_t)vnow[db][1]);
+        }
       }
     }
     if (!FP8) __builtin_amdgcn_sched_barrier(0);
@@ -769,7 +792,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 #pragma unroll
           for (int jj = 0; jj < NJ / 2; jj++) {
             const int j = hf * (NJ / 2) + jj;
-            kh[tb][jj] = *LDS_AT(u32x4, kaddr[j % NKA] + (SOFF + tb * HALF + (j / NKA) * (NKA * 64)));
+            kh[tb][jj] = *LDS_AT(u32x4, kb[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -869,12 +892,15 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     if constexpr (LATE_VREAD) {
       constexpr uint32_t HALF = 16 * G::ROW;
       constexpr int GB = 4;  // 16-column blocks per round of LDS reads
+      uint32_t vb[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) vb[i] = in_slot(vaddr[i], SOFF);
       auto read_group = [&](int g0, u32x4* dst) __attribute__((always_inline)) {
 #pragma unroll
         for (int e = 0; e < GB; e++) {
           const int db = g0 + e;
-          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + (db >> 3) * 256)));
-          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vaddr[db & 7] + (SOFF + HALF + (db >> 3) * 256)));
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vb[db & 7] + ((db >> 3) * 256)));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(s16x4, vb[db & 7] + (HALF + (db >> 3) * 256)));
           u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
           dst[e] = u32x4{l2[0], l2[1], h2[0], h2[1]};
         }
@@ -890,6 +916,29 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
           for (int rb = 0; rb < NRB; rb++) o_acc[rb][gi * GB + e] = Mma<QT>::run(vt[gi & 1][e], pk[rb], o_acc[rb][gi * GB + e]);
         __builtin_amdgcn_sched_barrier(0);  // keeps the rounds apart: at most two rounds of operands are live
       }
+      return;
+    }
+    if constexpr (LATE_VREAD8) {
+      constexpr int GB = 4;
+      auto read_group = [&](int g0, i32x2* dst) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < GB; e++) dst[e] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(i32x2, vaddr[g0 + e] + SOFF));
+      };
+      i32x2 vr[2][GB];
+      read_group(0, vr[0]);
+      __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int gi = 0; gi < NDB / GB; gi++) {
+        if (gi + 1 < NDB / GB) read_group((gi + 1) * GB, vr[(gi + 1) & 1]);
+#pragma unroll
+        for (int e = 0; e < GB; e++) {
+          const u32x4 vt = widen8<QT>((uint32_t)vr[gi & 1][e][0], (uint32_t)vr[gi & 1][e][1]);
+#pragma unroll
+          for (int rb = 0; rb < NRB; rb++) o_acc[rb][gi * GB + e] = Mma<QT>::run(vt, pk[rb], o_acc[rb][gi * GB + e]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_setprio(0);
       return;
     }
     if constexpr (SH && FP8) __builtin_amdgcn_s_setprio(1);
