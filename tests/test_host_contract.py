@@ -393,3 +393,17 @@ def test_benchmark_configurations_are_manifest_rows():
         assert entry["source"]["bench"] == "bench.py" and entry["source"].get("bench_manifest_driven") is True
     src = (ROOT / "bench.py").read_text()
     assert "load_workloads(" in src and "eval_roofline()" in src
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    """``bench.py --gpus N`` with N above 1 (or a multi-rank launch) exits non-zero before touching a device and says why."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parents[1] / "bench.py"
+    res = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0 and "one GPU" in res.stderr and res.stdout.strip() == ""
+    env = dict(__import__("os").environ, WORLD_SIZE="4")
+    res = subprocess.run([sys.executable, str(bench)], capture_output=True, text=True, timeout=120, env=env)
+    assert res.returncode != 0 and "one GPU" in res.stderr
