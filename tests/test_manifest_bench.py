@@ -87,6 +87,23 @@ def test_one_manifest_row_end_to_end(tmp_path):
         assert p["op"] == "GroupedQueryAttentionDecodePagedWithKVCacheFwdOp" and p["op_module"] == "tileops_amd.ops"
         assert float(p["tileops_latency_ms"]) > 0 and float(p["tileops_bandwidth_tbs"]) > 0 and 0 < float(p["tileops_hbm_frac"]) < 1
         assert abs(float(c.get("time")) * 1e3 - float(p["tileops_latency_ms"])) < 1e-3
+        # the same-device torch baseline of a paged row rides along under its own tag, and as the first baseline
+        if "softcap" not in c.get("name"):  # (torch's SDPA has no softcap: that row carries no baseline)
+            assert p["baseline_tag"] == "torch_sdpa" and float(p["torch_sdpa_latency_ms"]) > 0 and float(p["baseline_ratio"]) > 1
     log = (tmp_path / "profile_run.log").read_text()
     assert "## GroupedQueryAttentionDecodePagedWithKVCacheFwdOp" in log and "### tileops" in log and "serving-8b-p64" in log
+    assert "### torch_sdpa" in log
     assert torch.cuda.is_available()
+
+
+@pytest.mark.gpu
+def test_paged_torch_baseline_computes_what_the_op_computes():
+    """The baseline that paged rows are compared with (gather by block table, SDPA with a padding mask) agrees with the op
+    on ragged lengths and a permuted table -- a ratio against a wrong baseline would mean nothing."""
+    from tileops_amd.manifest import load_workloads
+
+    row = dict(next(r for r in load_workloads("GroupedQueryAttentionDecodePagedWithKVCacheFwdOp") if r["label"] == "serving-8b-p64"))
+    row.update(seqlen_range=[100, 4000], seed=4, kv_shape=[65536, 8, 128])
+    op, args, baseline = mb._paged_case(row, torch.bfloat16, torch.device("cuda", 0), False)
+    assert baseline is not None
+    torch.testing.assert_close(op(*args).float(), baseline().squeeze(2).float(), atol=2e-2, rtol=2e-2)

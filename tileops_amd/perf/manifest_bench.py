@@ -245,7 +245,32 @@ def _paged_case(row: dict, dtype: torch.dtype, device: torch.device, multi: bool
         args = wl.gen_inputs(device)
         lens = args[3]
     op.observe_call(lens, kv_dtype)
-    return op, args, None
+    return op, args, _paged_torch_baseline(op, args, row, page, multi, kv_dtype)
+
+
+def _paged_torch_baseline(op: Any, args: tuple, row: dict, page: int, multi: bool, kv_dtype: torch.dtype) -> Optional[Callable[[], Any]]:
+    """torch on the same device for a paged row: gather the pages each sequence addresses into a dense [B, max_len] cache
+    (one ``index_select`` per tensor on an index tensor built from the block table inside the call), then
+    ``F.scaled_dot_product_attention`` with a padding mask -- the role of the reference benchmark's SDPA baseline
+    (benchmarks/ops/attention/bench_gqa_decode_paged.py:21-66) without its per-page host loop.  16-bit caches, one query
+    token, no softcap, dense copy of at most 2 GiB; otherwise no baseline."""
+    q, k, v, lens, table = args[:5]
+    max_len = int(lens.max().item())
+    dense_bytes = 2 * q.shape[0] * max_len * k.shape[1] * k.shape[2] * k.element_size()
+    if multi or kv_dtype == FP8 or row.get("softcap") or dense_bytes > (2 << 30):
+        return None
+    import torch.nn.functional as F
+
+    def baseline():
+        t = torch.arange(max_len, device=q.device)
+        idx = table.long().gather(1, (t // page).expand(q.shape[0], -1)) * page + t % page  # [B, max_len] physical tokens
+        live = t[None, :] < lens[:, None]
+        idx = torch.where(live, idx, torch.zeros_like(idx))
+        kd = k.index_select(0, idx.reshape(-1)).view(q.shape[0], max_len, k.shape[1], k.shape[2]).transpose(1, 2)
+        vd = v.index_select(0, idx.reshape(-1)).view(q.shape[0], max_len, v.shape[1], v.shape[2]).transpose(1, 2)
+        return F.scaled_dot_product_attention(q.unsqueeze(2), kd, vd, attn_mask=live[:, None, None, :], scale=op.sm_scale, enable_gqa=True)
+
+    return baseline
 
 
 def _contiguous_case(row: dict, dtype: torch.dtype, device: torch.device):
