@@ -292,6 +292,28 @@ def test_multi_token_causal_chunk(kernel_key, fp8, q_len, is_causal):
         torch.testing.assert_close(out[:, i].float(), single(*args).float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_many_rows_merged_four_at_a_time(fp8, dim):
+    """More than 4096 rows in the call (40 sequences x 8 query tokens x 32 heads): the merge kernel's waves take four rows each
+    and have all their partial rows in flight together.  Ragged lengths so that sequences lie in one partition, in a few, or
+    are empty; the general kernel (its own merge) is the second opinion beside the oracle."""
+    require_gfx950()
+    g = torch.Generator().manual_seed(77)
+    B, q_len, H, H_kv = 40, 8, 32, 4
+    lens = [int(x) for x in torch.randint(q_len, 3000, (B,), generator=g)]
+    lens[3], lens[17], lens[39] = 0, q_len, 6000
+    case = _ragged_case(B, H, H_kv, dim, 64, lens, torch.bfloat16, q_len=q_len, fp8=fp8, seed=78)
+    op = MultiOp(B, q_len, H, H_kv, case[1].shape[0], dim, 64, is_causal=True)
+    _force(op, "gqa_decode_paged_mfma_kernel")
+    out = _run_and_compare(op, case, 64, 3e-2 if fp8 else 2e-2, is_causal=True)
+    other = MultiOp(B, q_len, H, H_kv, case[1].shape[0], dim, 64, is_causal=True)
+    _force(other, "gqa_decode_paged_kernel")
+    args = [None if t is None else t.to(DEV) for t in case]
+    args = tuple(args[:5]) + (() if args[5] is None else (args[5], args[6]))
+    torch.testing.assert_close(out.float(), other(*args).float(), atol=3e-2 if fp8 else 2e-2, rtol=3e-2 if fp8 else 2e-2)
+
+
 @pytest.mark.parametrize("dtype, fp8, tol", [(torch.bfloat16, False, 2e-2), (torch.float16, False, 2e-2), (torch.bfloat16, True, 3e-2),
                                              (torch.float16, True, 3e-2)])
 @pytest.mark.parametrize(

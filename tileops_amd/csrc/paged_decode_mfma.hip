@@ -1090,12 +1090,14 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 template <typename QT, int kCombineWaves>
 __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec,
                                             int wave);
+template <typename QT, int R>
+__device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int b, int row0, int row_end, int4 rec);
 
 // grid (ceil(heads_kv*rows / rows_per_wg), batch, halves of a 256-wide head): a workgroup takes rows_per_wg consecutive
 // rows of one sequence.  With thousands of rows per sequence (prefill chunks) most sequences lie inside one partition
 // and need no merge at all: the workgroup reads the sequence's record once and leaves, instead of one workgroup per row
 // doing so (131 072 of them took 28 us on an 8 x 512-row call).
-template <typename QT, int kCombineWaves>
+template <typename QT, int kCombineWaves, bool kManyRows = false>
 __global__ __launch_bounds__(256) void paged_decode_mfma_combine_kernel(const DecodeParams p, const int* __restrict__ ws_prefix, int rows_per_wg) {
   // always four waves: either they share one row at a time (kCombineWaves == 4) or each takes every fourth row of the
   // workgroup's range on its own (kCombineWaves == 1)
@@ -1107,6 +1109,12 @@ __global__ __launch_bounds__(256) void paged_decode_mfma_combine_kernel(const De
   const int row_end = min((int)(blockIdx.x + 1) * rows_per_wg, p.heads_kv * p.rows);
   const int phys_wave = uni(threadIdx.x >> 6);
   if constexpr (kCombineWaves == 1) {
+    constexpr int R = 4;
+    if (kManyRows && rows_per_wg >= 4 * R && rec.y >= 0 && rec.z - rec.y < 8 && (rec.w & 2) == 0) {
+      // many rows per workgroup, at most eight partials each: a wave takes R rows and has the loads of all of them in flight together
+      for (int row0 = blockIdx.x * rows_per_wg + phys_wave * R; row0 < row_end; row0 += 4 * R) combine_rows_at_once<QT, R>(p, b, row0, row_end, rec);
+      return;
+    }
     for (int row_all = blockIdx.x * rows_per_wg + phys_wave; row_all < row_end; row_all += 4)
       combine_row<QT, 1>(p, ws_prefix, red, b, row_all, rec, 0);
   } else {
@@ -1216,6 +1224,69 @@ __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __
   }
   const float inv = W > 0.f ? 1.0f / W : 0.f;
   store(acc0 * inv, acc1 * inv, W > 0.f ? M + log2f(W) : -INFINITY);
+}
+
+// R rows of one sequence merged by one wave, every load of every row issued before the first is consumed: with tens of
+// thousands of rows (eight query tokens x group 8 x 32 sequences) the merge kernel is otherwise two rounds of workgroups,
+// each a chain of three dependent reads.  At most eight partials per row, every partition owning tiles (the caller checks).
+template <typename QT, int R>
+__device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int b, int row0, int row_end, int4 rec) {
+  constexpr int PRE = 8;
+  const int lane = threadIdx.x & 63;
+  const int hd = p.dim;
+  const bool owns = 2 * lane < hd;
+  const int dl = owns ? 2 * lane + 128 * (int)blockIdx.z : 0;
+  const int p_first = rec.y, p_last = rec.z, n = p_last - p_first + 1;
+  const bool first_in_slot1 = (rec.w & 1) != 0;
+  const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
+  const int q_rows = p.cu_q ? q_len_of(p, b) * p.group : p.rows;
+  f32x2 rows[R][PRE];
+  float lse[R];
+  bool live[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const int row_all = min(row0 + r, row_end - 1);
+    const int kvh = row_all / p.rows;
+    live[r] = row0 + r < row_end && row_all - kvh * p.rows < q_rows;  // (packed queries: this sequence may have fewer rows)
+    auto slot_of = [&](int pp) { return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all; };
+#pragma unroll
+    for (int i = 0; i < PRE; i++) rows[r][i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + i, p_last)) * hd + dl);
+    lse[r] = lane < n ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    if (!live[r]) continue;
+    const int row_all = row0 + r;
+    const int kvh = row_all / p.rows, rr = row_all - kvh * p.rows;
+    const int s = rr / p.group, gi = rr - s * p.group;
+    const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
+    float M = lse[r];
+#pragma unroll
+    for (int m = 1; m < PRE; m <<= 1) M = fmaxf(M, __shfl_xor(M, m, 64));  // the first eight lanes hold the LSEs
+    M = __shfl(M, 0, 64);
+    const float w0 = (M != -INFINITY && lse[r] != -INFINITY) ? fast_exp2(lse[r] - M) : 0.f;
+    float W = w0;
+#pragma unroll
+    for (int m = 1; m < PRE; m <<= 1) W += __shfl_xor(W, m, 64);
+    W = __shfl(W, 0, 64);
+    float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+      const float wt = __shfl(w0, i, 64);
+      if (wt != 0.f) {  // an unwritten slot may hold anything, NaN included
+        acc0 = fmaf(wt, rows[r][i][0], acc0);
+        acc1 = fmaf(wt, rows[r][i][1], acc1);
+      }
+    }
+    const float inv = W > 0.f ? 1.0f / W : 0.f;
+    if (!owns) continue;
+    if (p.final_o) {
+      *(f32x2*)(p.final_o + orow * hd + dl) = f32x2{acc0 * inv, acc1 * inv};
+      if (lane == 0 && blockIdx.z == 0) p.final_lse[orow] = W > 0.f ? M + log2f(W) : -INFINITY;
+    } else {
+      *((uint32_t*)((uint16_t*)p.out + orow * hd) + (dl >> 1)) = Mma<QT>::pack(acc0 * inv, acc1 * inv);
+    }
+  }
 }
 
 // The same merge for calls whose sequences span very many partitions each (batch-1 long-context decode).
@@ -1388,12 +1459,15 @@ const char* launch_t4(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   const int rows_all = p.heads_kv * p.rows;
   const bool wide = (int64_t)p.n_parts > 64 * (int64_t)p.batch, four = !wide && (int64_t)p.n_parts > 8 * (int64_t)p.batch;
   int rows_per_wg = (wide || four) ? 1 : 4;
+  if (!wide && !four && (int64_t)rows_all * p.batch > 4096 && rows_all % 16 == 0) rows_per_wg = 16;  // four rows per wave, loaded together
   while ((int64_t)rows_all * p.batch / rows_per_wg > 8192 && rows_per_wg < 64) rows_per_wg *= 2;
   const dim3 cgrid((rows_all + rows_per_wg - 1) / rows_per_wg, p.batch, D > 128 ? 2 : 1);
   if (wide)
     hipLaunchKernelGGL((paged_decode_mfma_combine_wide_kernel<QT, 16>), cgrid, dim3(1024), 0, s, p, ws_prefix, rows_per_wg);
   else if (four)
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 4>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
+  else if (rows_per_wg >= 16)
+    hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1, true>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
   else
     hipLaunchKernelGGL((paged_decode_mfma_combine_kernel<QT, 1>), cgrid, dim3(256), 0, s, p, ws_prefix, rows_per_wg);
   e = hipGetLastError();
