@@ -7,6 +7,11 @@ CPU references timed on this box's host cores beside it; ``also`` holds the same
 configurations are workload rows of the op manifest (``load_workloads``); bytes and flops come from the op's
 ``eval_roofline()`` after it has seen the call.  Exit status 1 if any configuration misses its parity tolerance.
 
+Every configuration is measured in a process of its own (this one only starts them and joins their results): device
+memory that has been freed and allocated again inside one process reads 3-5 % slower than a fresh process's first
+allocations (measured: the FP8 configurations 99 -> 102 us and 335 -> 352 us after one ``empty_cache()``), and a serving
+process allocates its KV pool once, at start-up.
+
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--also c3,c4,c5] [--no-cpu]
 """
 
@@ -47,13 +52,13 @@ def _config(name: str):
 
 
 def _device_busy_ms(fn, flush, calls: int):
-    """Mean over ``calls`` flushed calls of the summed durations of this library's kernels in one call, from the torch
-    profiler's device events; None when the profiler delivers none."""
+    """Mean over ``calls`` flushed calls of the durations of this library's kernels in one call, from the torch profiler's
+    device events: (all kernels, attention kernel, merge kernel) in ms; None when the profiler delivers none."""
     try:
         import torch
         from torch.profiler import ProfilerActivity, profile
 
-        totals = []
+        totals, attn, merge = [], [], []
         for i in range(calls):
             flush(i)
             torch.cuda.synchronize()
@@ -64,10 +69,20 @@ def _device_busy_ms(fn, flush, calls: int):
             if not evs:
                 return None
             totals.append(sum(e.device_time for e in evs) / 1e3)
-        return sum(totals) / len(totals)
+            attn.append(sum(e.device_time for e in evs if "combine" not in e.name) / 1e3)
+            merge.append(sum(e.device_time for e in evs if "combine" in e.name) / 1e3)
+        n = len(totals)
+        return sum(totals) / n, sum(attn) / n, sum(merge) / n
     except Exception as exc:  # noqa: BLE001 - optional evidence; the timed figures above do not depend on it
         print(f"device-busy time not measured: {exc!r}", file=sys.stderr)
         return None
+
+
+def _spread(xs_ms: list[float]) -> dict:
+    """min / p10 / median / p90 / max of per-step times, in us."""
+    xs = sorted(x * 1e3 for x in xs_ms)
+    pick = lambda f: xs[min(len(xs) - 1, max(0, round(f * (len(xs) - 1))))]  # noqa: E731
+    return {"min": xs[0], "p10": pick(0.1), "median": statistics.median(xs), "p90": pick(0.9), "max": xs[-1]}
 
 
 def _timed_steps(fn, flush, steps: int) -> tuple[list[float], float]:
@@ -117,7 +132,8 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         flush_wr.fill_(i & 0xFF)
         flush_rd.max()
 
-    for _ in range(max(warmup, 1)):
+    for i in range(max(warmup, 1)):  # the flush kernels are part of what has to be warm
+        flush(i)
         out = op(*args)
     torch.cuda.synchronize()
     per_step_ms, wall = _timed_steps(lambda: op(*args), flush, steps)
@@ -132,25 +148,27 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     torch.cuda.synchronize()
     b2b_ms = s0.elapsed_time(s1) / steps
 
-    # The dominant (attention) kernel alone: launches that skip the merge of partial results, KREP back to back per
-    # event pair so that the few microseconds an event pair costs are spread over KREP launches.  Each launch streams
-    # far more than the 256 MB Infinity Cache holds, so a launch finds next to nothing of its predecessor cached.
-    KREP = 4
+    # The dominant (attention) kernel alone: launches that skip the merge of partial results.  The roofline figure is the
+    # cold one -- ONE launch per event pair, each after a cache flush, as a caller's launch finds the chip.  Beside it, for
+    # reference only, KREP launches back to back per event pair (warm address translation and metadata: 3-5 % kinder).
     kernel = next(iter(next(iter(op._kernel_roles.values())).values()))
     kernel.attention_kernel_only = True
+    k_cold_ms, _ = _timed_steps(lambda: op(*args), flush, steps)
+    kernel_ms = sum(k_cold_ms) / steps
+    KREP = 4
 
     def attention_only() -> None:
         for _ in range(KREP):
             op(*args)
 
-    k_ms, _ = _timed_steps(attention_only, flush, steps)
+    k_b2b_ms, _ = _timed_steps(attention_only, flush, steps)
     kernel.attention_kernel_only = False
-    kernel_ms = sum(k_ms) / (steps * KREP)
+    kernel_b2b_ms = sum(k_b2b_ms) / (steps * KREP)
     out = op(*args)  # complete output again for the parity check below
     torch.cuda.synchronize()
 
     # a whole call captured once in a HIP graph and replayed (what a serving loop does): no host launch gaps
-    graph_ms = graph_median_ms = None
+    graph_ms = graph_median_ms = graph8_ms = None
     if hasattr(op, "capture"):
         replay = op.capture(*args)
         for _ in range(3):
@@ -158,11 +176,27 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         g_ms, _ = _timed_steps(replay, flush, steps)
         graph_ms, graph_median_ms = sum(g_ms) / steps, statistics.median(g_ms)
         torch.cuda.synchronize()
+        # A serving loop's graph holds a whole model step, not one call: eight calls in ONE graph, replayed back to back, per
+        # call -- to be read against us_per_call_back_to_back (eager, also without flushes).  What a graph costs per LAUNCH
+        # (not per node) drops out of this figure and stays in the one-call figure above.
+        many = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(many):
+            for _ in range(8):
+                op(*args)
+        for _ in range(2):
+            many.replay()
+        s0.record()
+        for _ in range(max(steps // 4, 3)):
+            many.replay()
+        s1.record()
+        torch.cuda.synchronize()
+        graph8_ms = s0.elapsed_time(s1) / (max(steps // 4, 3) * 8)
+        del many
 
     # Device-busy time of a whole call: the sum of the durations of the kernels it launches (attention + merge), launch
     # latency and gaps excluded -- the quantity the reference's own timing protocol reports (its benchmarks take the
     # per-iteration device-busy time from the profiler, benchmarks/timing.py:527-585).  Ten flushed calls.
-    busy_ms = _device_busy_ms(lambda: op(*args), flush, 10)
+    busy = _device_busy_ms(lambda: op(*args), flush, 10)
 
     op.observe_call(inp.real_seqlen_kv, cfg.kv_dtype)
     flops, total_bytes = op.eval_roofline()
@@ -199,24 +233,34 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         # the whole call (attention kernel, merge of partial results where one is launched, launch gaps): mean and median of the
         # flushed steps, on the K/V (+ scale) bytes alone -- the figure the 70 % target is stated on -- and on all bytes
         "whole_call": {
-            "us_mean": ms * 1e3, "us_median": ms_median * 1e3,
+            "us_mean": ms * 1e3, "us_median": ms_median * 1e3, "us_spread": _spread(per_step_ms),
             "kv_read_gbs_mean": gbs(kv_read, ms), "kv_read_gbs_median": gbs(kv_read, ms_median),
             "kv_read_frac_of_peak_mean": gbs(kv_read, ms) / HBM_PEAK_GBS, "kv_read_frac_of_peak_median": gbs(kv_read, ms_median) / HBM_PEAK_GBS,
             "all_bytes_frac_of_peak_mean": gbs(total_bytes, ms) / HBM_PEAK_GBS,
         },
+        # the attention kernel alone, cold: one launch per HIP-event pair, each after a cache flush (mean of the steps)
         "attention_kernel_us": kernel_ms * 1e3,
-        # dominant kernel alone: algorithmic bytes of one launch / its own duration (events around the attention kernel only)
+        "attention_kernel_us_spread": _spread(k_cold_ms),
+        # the same kernel launched four times back to back per event pair (warm translation and metadata), for reference
+        "attention_kernel_us_back_to_back_x4": kernel_b2b_ms * 1e3,
+        "frac_back_to_back_x4": total_bytes / (kernel_b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        # dominant kernel alone: algorithmic bytes of one launch / its own cold duration
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic, "traffic_source": f"{TRAFFIC_SOURCE} (rocprofv3 FETCH_SIZE/WRITE_SIZE of an earlier profiler run, not counted in this run)"},
         "wall_s_timed_region": wall,
     }
-    if busy_ms is not None:
+    if busy is not None:
+        busy_ms, busy_attn_ms, busy_merge_ms = busy
         res["whole_call"].update({"us_device_busy_mean": busy_ms * 1e3, "kv_read_frac_of_peak_device_busy": gbs(kv_read, busy_ms) / HBM_PEAK_GBS})
+        # the profiler's own durations of the two kernels of a flushed call (no event pair involved)
+        res["profiler"] = {"attention_kernel_us": busy_attn_ms * 1e3, "merge_kernel_us": busy_merge_ms * 1e3,
+                           "attention_kernel_frac": total_bytes / (busy_attn_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if busy_attn_ms else None}
     if graph_ms is not None:
         res["whole_call"].update({
             "us_graph_mean": graph_ms * 1e3, "us_graph_median": graph_median_ms * 1e3,
             "kv_read_frac_of_peak_graph_mean": gbs(kv_read, graph_ms) / HBM_PEAK_GBS,
             "kv_read_frac_of_peak_graph_median": gbs(kv_read, graph_median_ms) / HBM_PEAK_GBS,
+            "us_per_call_in_a_graph_of_8_back_to_back": graph8_ms * 1e3,
         })
     if cfg.q_len * (cfg.heads // cfg.heads_kv) >= 16:
         # enough query rows per kv head for the products to be dense matrix work: report the matrix rate beside the bandwidth
@@ -261,6 +305,32 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     return res
 
 
+def _measure_here(name: str, a) -> dict:
+    import torch
+
+    from tileops_amd import native
+
+    native.require_gfx950(torch.device("cuda", 0))
+    return _run_config(name, a.steps, a.warmup, not a.no_cpu, a.kernel)
+
+
+def _measure_in_child(name: str, a) -> dict:
+    """One configuration in a process of its own.  This process has not touched the GPU (it imports no torch), so the
+    child is an ordinary fresh program; its stderr passes through, its last stdout line is the result."""
+    import subprocess
+
+    cmd = [sys.executable, str(Path(__file__).resolve()), "--child", name, "--steps", str(a.steps), "--warmup", str(a.warmup)]
+    if a.no_cpu:
+        cmd.append("--no-cpu")
+    if a.kernel:
+        cmd += ["--kernel", a.kernel]
+    done = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)
+    lines = [ln for ln in done.stdout.splitlines() if ln.startswith("{")]
+    if done.returncode != 0 or not lines:
+        sys.exit(f"measuring {name} failed (exit status {done.returncode}): {done.stdout[-2000:]}")
+    return json.loads(lines[-1])
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -270,26 +340,34 @@ def main() -> None:
     ap.add_argument("--also", default="c3,c4,c5", help="comma-separated extra configurations reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU reference legs (and with them the parity check)")
     ap.add_argument("--kernel", default=None, choices=[None, "gqa_decode_paged_kernel", "gqa_decode_paged_mfma_kernel"])
+    ap.add_argument("--in-process", action="store_true",
+                    help="measure every configuration in this process, one after the other (their pools then land in memory that "
+                         "was freed and allocated again: 3-5 %% slower from the second configuration on)")
+    ap.add_argument("--child", default=None, choices=["c2", "c3", "c4", "c5"], help=argparse.SUPPRESS)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies, so a hardware-counter pass has a kernel of known traffic to scale by")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the path is single-GPU by construction (every (sequence, kv-head) is independent); "
                  "run with --gpus 1")
-    import torch
-
-    from tileops_amd import native
-
-    native.require_gfx950(torch.device("cuda", 0))
-    main_res = _run_config(a.config, a.steps, a.warmup, not a.no_cpu, a.kernel)
-    also = [_run_config(n, a.steps, a.warmup, not a.no_cpu, a.kernel) for n in a.also.split(",") if n and n != a.config]
+    names = [a.config] + [n for n in a.also.split(",") if n and n != a.config]
+    if a.child:
+        # one configuration, in this process; the result goes to the parent as one JSON line
+        print(json.dumps(_measure_here(a.child, a)))
+        return
+    if len(names) == 1 or a.in_process:
+        results = [_measure_here(n, a) for n in names]  # (a profiler run names one configuration and lands here)
+    else:
+        results = [_measure_in_child(n, a) for n in names]
+    main_res, also = results[0], results[1:]
     fp8 = a.config != "c2"
     line = {
         "metric": "GQA paged-decode us/call (achieved HBM GB/s and fraction of the 8 TB/s peak under 'roofline')",
         "value": main_res["us_per_call"], "unit": "us/call", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": main_res["us_per_call"] / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3fn KV / bf16 Q, fp32 accumulate" if fp8 else "bf16",
-        "data": "synthetic", "config": {"workload": main_res["workload"], "kernel": main_res["kernel"]},
+        "data": "synthetic", "config": {"workload": main_res["workload"], "kernel": main_res["kernel"],
+                                        "process": "one per configuration" if len(names) > 1 and not a.in_process else "this one"},
         "roofline": main_res["roofline"],
     }
     for key in ("cpu_baseline", "cpu_baseline_sdpa_math", "parity", "mfma"):
@@ -297,7 +375,9 @@ def main() -> None:
             line[key] = main_res[key]
     line["detail"] = {k: v for k, v in main_res.items() if k not in ("roofline", "cpu_baseline", "cpu_baseline_sdpa_math", "parity", "mfma", "workload")}
     line["also"] = also
-    if a.copy_calibration:
+    if a.copy_calibration and (len(names) == 1 or a.in_process):
+        import torch
+
         src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(3):

@@ -60,11 +60,15 @@ const char* mi355_last_error(void);
  *
  *   max_blocks_per_seq : width of block_table actually usable (>= ceil(max context / page_size))
  *   num_split_in       : 0 = choose; > 0 = upper bound on KV splits per sequence (generic kernel) /
- *                        ignored by the MFMA kernel, which partitions the KV tile stream evenly over
- *                        all compute units instead
+ *                        number of equal ranges the MFMA kernel cuts the KV tile stream into (at most 4096;
+ *                        0 = one range per wave the chip holds, which is what measures best -- the knob is
+ *                        there for the kernel class's autotuner)
  *   kernel             : MI355_KERNEL_*
  * Outputs: *workspace_bytes (may be 0), *num_split_out (splits per sequence the generic kernel will
  * use at most; number of stream partitions for the MFMA kernel), *kernel_out (the kernel AUTO resolved to).
+ * The query touches no device and initialises no HIP runtime: with num_split_in == 0 it plans for the 256 compute
+ * units of an MI355X.  A launch on a device with fewer compute units uses fewer partitions and so never needs more
+ * workspace than the query reported; pass num_split_out back as num_split to get exactly the plan that was sized.
  */
 int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_kv, int dim, int page_size,
                                      int64_t max_blocks_per_seq, int q_dtype, int kv_dtype, int num_split_in,
@@ -115,6 +119,13 @@ int mi355_gqa_paged_decode(const void* q, const void* k, const void* v, const fl
  * kernel's plan grows with batch x splits and may not);
  * all calls on one GPU share that GPU's array, so two calls that overlap in time on one GPU (different streams) race --
  * keep such calls on one stream, or use mi355_gqa_paged_decode with separate workspaces.  Arguments as there.
+ * Under graph capture: the first call on a device (of a process, per kernel instance it selects) does one-time set-up
+ * that is not stream work -- it asks the runtime for the array's device address and raises the kernels' LDS limit -- and
+ * must not itself be captured.  Make one ordinary call of the same shape on that device first, then capture; captured
+ * calls enqueue the two kernels and nothing else (no memset node), and replays pick up changed cache contents, lengths
+ * and block tables in place.
+ * Cost: the array is part of the library's device image, so every process that loads the library holds 80 MiB on every
+ * GPU it initialises, whether or not it ever calls this entry point (16 processes on one GPU: 1.3 GB).
  */
 int mi355_gqa_paged_decode_static(const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
                                   const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride, void* out,

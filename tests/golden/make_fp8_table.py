@@ -1,6 +1,7 @@
 """Writes tests/golden/fp8_e4m3fn_table.json: the 256 values of OCP FP8 E4M3FN as torch.float8_e4m3fn decodes
-them (torch is a library present on every box; the reference is not involved), plus the fp32 values at which
-rounding switches between adjacent finite codes.  Run once: ``python tests/golden/make_fp8_table.py``."""
+them, as fp32 bit patterns (null for the two NaN codes).  torch is a library present on every box; the reference is
+not involved.  The encoder's rounding is pinned elsewhere (tests/test_oracle_fp8.py: a dense grid, the midpoints
+between neighbouring codes included, against torch's own cast).  Run once: ``python tests/golden/make_fp8_table.py``."""
 
 import json
 import struct

@@ -89,10 +89,10 @@ def test_one_manifest_row_end_to_end(tmp_path):
         assert abs(float(c.get("time")) * 1e3 - float(p["tileops_latency_ms"])) < 1e-3
         # the same-device torch baseline of a paged row rides along under its own tag, and as the first baseline
         if "softcap" not in c.get("name"):  # (torch's SDPA has no softcap: that row carries no baseline)
-            assert p["baseline_tag"] == "torch_sdpa" and float(p["torch_sdpa_latency_ms"]) > 0 and float(p["baseline_ratio"]) > 1
+            assert p["baseline_tag"] == "torch_gather_sdpa" and float(p["torch_gather_sdpa_latency_ms"]) > 0 and float(p["baseline_ratio"]) > 1
     log = (tmp_path / "profile_run.log").read_text()
     assert "## GroupedQueryAttentionDecodePagedWithKVCacheFwdOp" in log and "### tileops" in log and "serving-8b-p64" in log
-    assert "### torch_sdpa" in log
+    assert "### torch_gather_sdpa" in log
     assert torch.cuda.is_available()
 
 

@@ -83,8 +83,14 @@ struct Plan {
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
+constexpr int kPlanCuCount = 256;    // MI355X: 8 XCDs x 32 compute units
+constexpr int kMaxMfmaParts = 4096;  // the kernel's 32-bit partition arithmetic holds up to here
+
+// for_launch: the call is about to run on the current device, whose compute-unit count sizes the MFMA kernel's partition
+// count (never more than the 256 of an MI355X, which is what a workspace query plans for without touching any device, so a
+// workspace sized by the query always holds the launch's plan).
 int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_size, int64_t max_blocks_per_seq, int q_dtype,
-              int kv_dtype, float softcap, int num_split_in, int kernel, Plan* plan) {
+              int kv_dtype, float softcap, int num_split_in, int kernel, Plan* plan, bool for_launch = false) {
   if (max_blocks_per_seq < 0) return fail(MI355_EINVAL, "max_blocks_per_seq must be non-negative");
   if (num_split_in < 0) return fail(MI355_EINVAL, "num_split must be non-negative, got %d", num_split_in);
   const int rows = q_len * (heads / heads_kv);
@@ -112,7 +118,9 @@ int make_plan(int batch, int q_len, int heads, int heads_kv, int dim, int page_s
   } else {
     plan->max_splits = 0;
     plan->split_tokens = 0;
-    plan->n_parts = mfma_num_parts(heads_kv, rows, dim, kv_dtype);
+    // num_split > 0 fixes the partition count (what the kernel class's autotuner varies); 0 = one range per resident wave
+    const int cus = for_launch ? (device_cu_count() < kPlanCuCount ? device_cu_count() : kPlanCuCount) : kPlanCuCount;
+    plan->n_parts = num_split_in > 0 ? (num_split_in < kMaxMfmaParts ? num_split_in : kMaxMfmaParts) : mfma_num_parts(heads_kv, rows, dim, kv_dtype, cus);
     size_t total = mfma_workspace_bytes(plan->n_parts, heads_kv, rows, dim, batch);
     plan->part_o_bytes = total;  // the MFMA launcher lays out its own workspace
     plan->part_lse_bytes = 0;
@@ -148,7 +156,7 @@ int run_decode(const void* q, const void* k, const void* v, const float* k_scale
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(MI355_EINVAL, "q, k, v and out must be 16-byte aligned");
   Plan plan;
-  int rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan);
+  int rc = make_plan(batch, q_len, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kv_dtype, softcap, num_split, kernel, &plan, true);
   if (rc) return rc;
   const size_t need = plan.part_o_bytes + plan.part_lse_bytes;
   if (need > 0) {

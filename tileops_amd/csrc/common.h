@@ -78,17 +78,31 @@ __device__ __forceinline__ int64_t q_row0_of(const DecodeParams& p, int b) { ret
 // has query rows, the other branch leaves the load formally outstanding, and the compiler protects the next write of
 // that register -- wherever it is, in practice an LDS read of the tile loop -- with a vmcnt(0) that drains every
 // prefetch on every tile (measured: 146 -> 167 us on the eight-query-token FP8 workload).
-template <bool kLand = false>
-__device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) {
-  int len = p.seqlens ? p.seqlens[b] : p.uniform_len;
-  int ql = 1;
-  if (p.cu_q) ql = p.cu_q[b + 1] - p.cu_q[b];
-  if constexpr (kLand) asm volatile("" : "+v"(len), "+v"(ql));
+// The two loads of a length, apart from what is made of them, so that a caller can request them early and use them late.
+struct RawSeqLen {
+  int len, ql;
+};
+__device__ __forceinline__ RawSeqLen seq_len_load(const DecodeParams& p, int b) {
+  RawSeqLen r;
+  r.len = p.seqlens ? p.seqlens[b] : p.uniform_len;
+  r.ql = 1;
+  if (p.cu_q) r.ql = p.cu_q[b + 1] - p.cu_q[b];
+  return r;
+}
+__device__ __forceinline__ int seq_len_finish(const DecodeParams& p, RawSeqLen r) {
+  int len = r.len;
   if (p.cu_q) {
-    if (ql <= 0) return 0;  // no query rows: nothing to compute, the sequence contributes no tile
-    if (p.len_excludes_new) len += ql;
+    if (r.ql <= 0) return 0;  // no query rows: nothing to compute, the sequence contributes no tile
+    // (saturating: a corrupt length near INT_MAX must end up clamped to max_len, not wrapped to a negative number)
+    if (p.len_excludes_new) len = len > p.max_len - r.ql ? p.max_len : len + r.ql;
   }
   return min(max(len, 0), p.max_len);
+}
+template <bool kLand = false>
+__device__ __forceinline__ int seq_len_of(const DecodeParams& p, int b) {
+  RawSeqLen r = seq_len_load(p, b);
+  if constexpr (kLand) asm volatile("" : "+v"(r.len), "+v"(r.ql));
+  return seq_len_finish(p, r);
 }
 
 // Number of KV splits of one sequence and the (tile-aligned) tokens per split, generic kernel.
@@ -108,11 +122,11 @@ __host__ __device__ inline void split_geometry(int len, int split_tokens, int ma
 const char* launch_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
 const char* launch_generic_combine(const DecodeParams& p, int q_dtype, hipStream_t s);
 bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, int q_dtype, int kv_dtype, float softcap);
-int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype);
+int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype, int compute_units);
 size_t mfma_workspace_bytes(int n_parts, int heads_kv, int rows, int dim, int batch);
 const char* launch_mfma(const DecodeParams& p, int q_dtype, int kv_dtype, bool skip_combine, hipStream_t s);
-// Compute units of the current device (256 on MI355X; that figure also when no device is visible, so that workspace
-// plans can be made on a host without a GPU).  Asked once per device.
+// Compute units of the current device (256 on MI355X; that figure also when no device is visible).  Asked once per
+// device, and only by entry points that launch: workspace queries plan for 256 and touch no device.
 int device_cu_count();
 const char* launch_gather_probe(const void* cache, const int32_t* seqlens, const int32_t* block_table, int64_t bt_row_stride,
                                 void* dense_out, int batch, int64_t max_len, int64_t row_bytes, int page_size,

@@ -179,10 +179,21 @@ __device__ __forceinline__ float group_sum(float x) {
 // below 2^-126 may flush to zero, which is what a softmax weight that small should be).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Inclusive prefix sum over the 64 lanes on the data-parallel-primitive path (no LDS crossbar): four shifts inside each row
+// of 16 lanes, then lane 15 of rows 0 and 2 added to rows 1 and 3, then lane 31 to rows 2 and 3.
+__device__ __forceinline__ int wave_incl_scan(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
 __device__ __forceinline__ int units_of(int len) { return (len + kCT - 1) / kCT; }
 
-// Which partition holds global tile index u, for bounds u0(p) = floor(p*T/NP).
-__device__ __forceinline__ int part_of(int64_t u, int64_t T, int64_t NP) { return (int)(((u + 1) * NP - 1) / T); }
+// Partition bounds u0(p) = floor(p*T/NP) (the merge kernels; the attention kernel forms the same numbers in 32 bits).
 __device__ __forceinline__ int part_begin(int64_t p, int64_t T, int64_t NP) { return (int)(p * T / NP); }
 
 // Position in the tile stream: sequence b, tile j of nt, plus the logical page / in-page offset of tile j.
@@ -293,76 +304,99 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   const int part = uni(part_);
   const int kvh = uni(kvh_);
   const int rg = uni(rg_);
-  const int64_t NP = p.n_parts;
   const bool ps16 = p.page_size == 16;
 
   // ---- tile-stream bookkeeping: total tiles, this partition's range, first sequence of the range ------
+  // One pass over the lengths (the first 64 stay in registers: with up to 64 sequences nothing is loaded twice), prefix
+  // sums inside the wave on the data-parallel-primitive path, partition bounds in 32-bit arithmetic.  Everything a wave
+  // does before its first K/V fetch is latency that no other wave of the compute unit hides: all of them are here too.
   int T = 0;
+  int lens0 = 0, n0 = 0, incl0 = 0;
   for (int base = 0; base < p.batch; base += 64) {
-    int b = base + lane;
-    int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) n += __shfl_xor(n, m, 64);
-    T += n;
+    const int b = base + lane;
+    const int len = b < p.batch ? seq_len_of<true>(p, b) : 0;
+    const int n = units_of(len);
+    const int incl = wave_incl_scan(n);
+    if (base == 0) {
+      lens0 = len;
+      n0 = n;
+      incl0 = incl;
+    }
+    T += __builtin_amdgcn_readlane(incl, 63);
   }
   T = uni(T);
+  // bounds u0(p) = floor(p*T/NP) = p*(T/NP) + floor(p*(T%NP)/NP): the second product stays below NP^2 <= 2^24
+  const uint32_t NPu = (uint32_t)p.n_parts, Tq = (uint32_t)T / NPu, Tr = (uint32_t)T - Tq * NPu;
+  auto bound = [&](uint32_t pp) __attribute__((always_inline)) -> int { return (int)(pp * Tq + (pp * Tr) / NPu); };
   if (gw == 0) {
     // Per-sequence record for the combine kernel: {first tile, first partition, last partition, whether the
     // first partition holds this sequence in its second partial slot}.  Entry [batch] = {T, 0, 0, 0}.
+    // Partition of tile u = the largest p with bound(p) <= u: a float estimate, off by at most one, put right by bound().
+    const float np_over_t = (float)NPu / (float)(T > 0 ? T : 1);
+    auto owner = [&](int u) __attribute__((always_inline)) -> int {
+      int pp = min(max((int)((float)(u + 1) * np_over_t) - 1, 0), (int)NPu - 1);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        if (bound((uint32_t)pp) > u) --pp;
+#pragma unroll
+      for (int i = 0; i < 3; i++)
+        if (pp + 1 < (int)NPu && bound((uint32_t)pp + 1) <= u) ++pp;
+      return pp;
+    };
     int carry = 0;
     for (int base = 0; base < p.batch; base += 64) {
-      int b = base + lane;
-      int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
-      int incl = n;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        int t = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += t;
+      const int b = base + lane;
+      int n = n0, incl = incl0;
+      if (base > 0) {
+        n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
+        incl = wave_incl_scan(n);
       }
       if (b < p.batch) {
         int pre = carry + incl - n;
         int4 rec = {pre, -1, -1, 0};  // y < 0 marks an empty sequence
         if (n > 0) {
-          rec.y = part_of(pre, T, NP);
-          rec.z = part_of(pre + n - 1, T, NP);
-          rec.w = (part_begin(rec.y, T, NP) != pre ? 1 : 0) | (T < NP ? 2 : 0);  // bit 1: some partitions own no tile
+          rec.y = owner(pre);
+          rec.z = owner(pre + n - 1);
+          rec.w = (bound((uint32_t)rec.y) != pre ? 1 : 0) | (T < (int)NPu ? 2 : 0);  // bit 1: some partitions own no tile
         }
         ((int4*)ws_prefix)[b] = rec;
       }
-      carry += __shfl(incl, 63, 64);
+      carry += __builtin_amdgcn_readlane(incl, 63);
     }
     if (lane == 0) ((int4*)ws_prefix)[p.batch] = int4{T, 0, 0, 0};
   }
   if (part >= p.n_parts || T == 0) return;
-  const int u0 = part_begin(part, T, NP), u1 = part_begin(part + 1, T, NP);
+  const int u0 = bound((uint32_t)part), u1 = bound((uint32_t)part + 1);
   const int n_units = u1 - u0;
   if (n_units <= 0) return;
 
   Cursor start;
   {
     int carry = 0, b0 = -1, pre0 = 0;
+    start.lens = lens0;
+    start.lens_base = 0;
     for (int base = 0; base < p.batch && b0 < 0; base += 64) {
-      int b = base + lane;
-      int n = b < p.batch ? units_of(seq_len_of<true>(p, b)) : 0;
-      int incl = n;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        int t = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += t;
+      const int b = base + lane;
+      int len = lens0, n = n0, incl = incl0;
+      if (base > 0) {
+        len = b < p.batch ? seq_len_of<true>(p, b) : 0;
+        n = units_of(len);
+        incl = wave_incl_scan(n);
       }
-      uint64_t hit = __ballot(carry + incl > u0);
+      const uint64_t hit = __ballot(carry + incl > u0);
       if (hit) {
-        int idx = __ffsll((unsigned long long)hit) - 1;
+        const int idx = uni(__ffsll((unsigned long long)hit) - 1);
         b0 = base + idx;
-        pre0 = carry + __shfl(incl - n, idx, 64);
+        pre0 = carry + __builtin_amdgcn_readlane(incl - n, idx);
+        start.lens = len;  // lane l = sequence base + l: the cursor starts on registers already here
+        start.lens_base = base;
       }
-      carry += __shfl(incl, 63, 64);
+      carry += __builtin_amdgcn_readlane(incl, 63);
     }
     b0 = uni(b0);
     pre0 = uni(pre0);
     start.b = b0;
-    cursor_load_lens(start, p, b0);
-    start.len = __builtin_amdgcn_readlane(start.lens, 0);
+    start.len = __builtin_amdgcn_readlane(start.lens, b0 - start.lens_base);
     start.nt = units_of(start.len);
     start.j = u0 - pre0;
     if (ps16) {
@@ -1537,14 +1571,14 @@ bool mfma_supported(int q_len, int heads, int heads_kv, int dim, int page_size, 
 
 // Number of equal ranges the tile stream is cut into: one wave per (range, kv head, row group), sized so
 // that every compute unit holds one (16-bit KV) or two (fp8 KV, half the LDS per stage) workgroups.
-int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype) {
+int mfma_num_parts(int heads_kv, int rows, int dim, int kv_dtype, int compute_units) {
   const bool fp8 = kv_dtype == MI355_DT_FP8_E4M3FN;
   const int nrb = row_blocks_for(rows, dim), shw = ring_waves_for(rows, nrb, max_ring_for(dim, fp8));
   const int n_rg = ring_row_groups(rows, nrb, shw);
   // resident waves per CU: eight with 128-byte rows (fp8, or head dim 64; LDS-limited) and for shared rings (accumulators in ordinary
   // vector registers, two waves per SIMD), four for unshared 16-bit waves (LDS-limited: 2 x 16 KiB stages each)
   const int waves_per_cu = dim == 256 ? (shw == 8 ? 8 : (shw > 1 || fp8) ? 4 : 2) : ((fp8 || dim == 64 || shw > 1) ? 8 : 4);
-  const int64_t waves = (int64_t)device_cu_count() * waves_per_cu;
+  const int64_t waves = (int64_t)compute_units * waves_per_cu;
   int64_t parts = waves / ((int64_t)heads_kv * n_rg);
   return parts < 1 ? 1 : (int)parts;
 }

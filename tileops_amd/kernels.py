@@ -21,6 +21,7 @@ from typing import Any, Optional
 
 import torch
 
+from . import custom_ops as _custom_ops  # noqa: F401 - registers torch.ops.tileops_amd.*
 from . import native
 
 __all__ = [
@@ -28,7 +29,7 @@ __all__ = [
     "GQADecodePagedMfmaKernel", "GQAPrefillPagedWithFP8KVCacheFwdKernel", "GQAPrefillPagedWithKVCacheFwdKernel",
     "GQAPrefillPagedWithKVCacheRopeFwdKernel", "Kernel",
     "PAGED_DECODE_KEYS", "PAGED_PREFILL_KEYS", "PrefillCall",
-    "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch",
+    "gqa_decode_paged_block_n", "gqa_decode_paged_block_ns", "get_arch", "mfma_kernel_serves",
 ]
 
 #: Dispatch keys of the paged decode ops, in no particular order (selection never reads the order).
@@ -42,13 +43,19 @@ DECODE_KEYS = ("gqa_decode_kernel", "gqa_decode_mfma_kernel")
 GFX950_ARCH = 95  # torch.cuda.get_device_capability() == (9, 5) on gfx950
 
 
-@functools.lru_cache(maxsize=None)
-def get_arch(device_index: Optional[int] = None) -> Optional[int]:
-    """major*10+minor of a ROCm device, or None when no GPU is visible."""
+@torch._dynamo.assume_constant_result
+def _arch_of(device_index: Optional[int]) -> Optional[int]:
+    # (a constant to the tracer: asked once while a graph is being built, never a node of it)
     if not torch.cuda.is_available():
         return None
     major, minor = torch.cuda.get_device_capability(device_index)
     return major * 10 + minor
+
+
+@functools.lru_cache(maxsize=None)
+def get_arch(device_index: Optional[int] = None) -> Optional[int]:
+    """major*10+minor of a ROCm device, or None when no GPU is visible."""
+    return _arch_of(device_index)
 
 
 def _as_torch_dtype(dtype: Any) -> torch.dtype:
@@ -80,6 +87,17 @@ class AttentionCall:
     @property
     def group(self) -> int:
         return self.heads // self.heads_kv
+
+
+def mfma_kernel_serves(dim: int, page_size: int, dtype: torch.dtype, kv_dtype: torch.dtype) -> bool:
+    """The region the library's MFMA kernel serves (``mfma_supported`` in csrc/paged_decode_mfma.hip; a test holds the
+    two together): head dim 64, 128 or 256, pages of 16 tokens or a multiple of 32, a 16-bit cache of the query's type or
+    an FP8-e4m3fn cache.  Stated here in plain Python so that kernel selection is traceable by ``torch.compile``."""
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    if kv_dtype != torch.float8_e4m3fn and kv_dtype != dtype:
+        return False
+    return dim in (64, 128, 256) and (page_size == 16 or (page_size > 0 and page_size % 32 == 0))
 
 
 def gqa_decode_paged_block_ns(page_size: int) -> tuple[int, ...]:
@@ -203,7 +221,6 @@ class GQADecodePagedKernel(Kernel):
             raise ValueError("page_size must be positive")
         if self.seqlen_kv % self.page_size != 0:
             raise ValueError("seqlen_kv must be divisible by page_size")
-        self._plans: dict[tuple[int, int], tuple[int, int]] = {}
         self.init_config(config, tune)
 
     # -- config ----------------------------------------------------------------------------------------
@@ -248,16 +265,6 @@ class GQADecodePagedKernel(Kernel):
         self.config = best
 
     # -- launch ----------------------------------------------------------------------------------------
-    def _plan(self, max_blocks_per_seq: int) -> tuple[int, int]:
-        key = (max_blocks_per_seq, int(self.config.get("num_split", 0)))
-        plan = self._plans.get(key)
-        if plan is None:
-            nbytes, nsplit, _ = native.decode_workspace(
-                self.batch, self.q_len, self.heads, self.groups, self.dim, self.page_size, max_blocks_per_seq,
-                self.dtype, self.kv_dtype, key[1], self._native_kernel)
-            plan = self._plans[key] = (nbytes, nsplit)
-        return plan
-
     #: Measurement aid: when True, ``forward`` launches the attention kernel alone (no combine), so a benchmark
     #: can time the dominant kernel by itself.  The returned tensor is then incomplete.
     attention_kernel_only: bool = False
@@ -265,17 +272,13 @@ class GQADecodePagedKernel(Kernel):
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: torch.Tensor,
                 block_table: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
                 v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-        native.require_gfx950(q.device)
-        nbytes, nsplit = self._plan(block_table.shape[1])
-        out = torch.empty_like(q)
-        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
-        native.paged_decode(
-            q, k, v, k_scale, v_scale, real_seqlen_kv, block_table, out, workspace,
-            batch=self.batch, q_len=self.q_len, heads=self.heads, heads_kv=self.groups, dim=self.dim,
-            page_size=self.page_size, sm_scale=self.sm_scale, softcap=self.softcap, causal=self.is_causal,
-            num_split=nsplit,
-            kernel=self._native_kernel | (native.KERNEL_FLAG_SKIP_COMBINE if self.attention_kernel_only else 0))
-        return out
+        # one registered operator (custom_ops.py): output and workspace are allocated inside it, so a compiled caller
+        # sees a single graph node
+        return torch.ops.tileops_amd.gqa_paged_decode(
+            q, k, v, real_seqlen_kv, block_table, k_scale, v_scale, self.q_len, self.heads, self.groups, self.dim,
+            self.page_size, float(self.sm_scale), float(self.softcap), bool(self.is_causal),
+            int(self.config.get("num_split", 0) or 0),
+            self._native_kernel | (native.KERNEL_FLAG_SKIP_COMBINE if self.attention_kernel_only else 0))
 
 
 class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
@@ -288,12 +291,7 @@ class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
 
     @classmethod
     def applies(cls, call: AttentionCall) -> bool:
-        try:
-            native.decode_workspace(call.batch, call.q_len, call.heads, call.heads_kv, call.dim, call.page_size, 1,
-                                    call.dtype, call.kv_dtype or call.dtype, 0, native.KERNEL_MFMA)
-        except (NotImplementedError, ValueError):
-            return False
-        return True
+        return mfma_kernel_serves(call.dim, call.page_size, call.dtype, call.kv_dtype or call.dtype)
 
     @property
     def default_config(self) -> dict[str, Any]:
@@ -301,7 +299,16 @@ class GQADecodePagedMfmaKernel(GQADecodePagedKernel):
 
     @property
     def autotune_configs(self) -> list[dict]:
-        return [dict(self.default_config)]
+        """``num_split`` is the number of equal ranges the KV tile stream is cut into (0 = one per resident wave, the
+        library's own choice).  The candidates are that choice and whole multiples / halves of it: the grid then stays a
+        whole number of rounds over the compute units (a count in between leaves a round part-filled and measured
+        25-30 % slower on the Llama-3-8B shapes; two rounds of half-length ranges cost 3-7 % there, and pay only where
+        the sequences are too few and too uneven for one round to balance)."""
+        block_n = gqa_decode_paged_block_n(self.page_size)
+        _, auto, _ = native.decode_workspace(self.batch, self.q_len, self.heads, self.groups, self.dim, self.page_size, 1,
+                                             self.dtype, self.kv_dtype, 0, native.KERNEL_MFMA)
+        counts = [0] + [n for n in (auto // 2, 2 * auto, 4 * auto) if n >= 1]
+        return [{"block_N": block_n, "num_split": n} for n in counts]
 
 
 class GQADecodeKernel(Kernel):
@@ -333,7 +340,6 @@ class GQADecodeKernel(Kernel):
             raise ValueError("heads must be divisible by groups")
         if self.seqlen_kv <= 0:
             raise ValueError("seqlen_kv must be positive")
-        self._plans: dict[int, tuple[int, int]] = {}
         self.init_config(config, tune)
 
     def _default_num_split(self) -> int:
@@ -377,29 +383,13 @@ class GQADecodeKernel(Kernel):
                 best, best_ms = dict(cfg), ms
         self.config = best
 
-    def _plan(self) -> tuple[int, int]:
-        key = int(self.config.get("num_split", 0))
-        plan = self._plans.get(key)
-        if plan is None:
-            nbytes, nsplit, _ = native.contiguous_decode_workspace(
-                self.batch, 1, self.heads, self.groups, self.dim, self.seqlen_kv, self.dtype, self.kv_dtype, key,
-                self._native_kernel)
-            plan = self._plans[key] = (nbytes, nsplit)
-        return plan
-
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, real_seqlen_kv: int,
                 k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-        native.require_gfx950(q.device)
         if real_seqlen_kv > self.seqlen_kv:
             raise ValueError(f"real_seqlen_kv={real_seqlen_kv} exceeds the seqlen_kv={self.seqlen_kv} this kernel was built for")
-        nbytes, nsplit = self._plan()
-        out = torch.empty_like(q)
-        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
-        native.contiguous_decode(
-            q, k, v, k_scale, v_scale, out, workspace, batch=self.batch, q_len=1, heads=self.heads, heads_kv=self.groups,
-            dim=self.dim, real_seqlen_kv=real_seqlen_kv, sm_scale=self.sm_scale, softcap=self.softcap, causal=True,
-            num_split=nsplit, kernel=self._native_kernel)
-        return out
+        return torch.ops.tileops_amd.gqa_decode(
+            q, k, v, k_scale, v_scale, int(real_seqlen_kv), self.heads, self.groups, self.dim, float(self.sm_scale),
+            float(self.softcap), True, int(self.config.get("num_split", 0) or 0), self._native_kernel)
 
 
 class GQADecodeMfmaKernel(GQADecodeKernel):
@@ -412,13 +402,7 @@ class GQADecodeMfmaKernel(GQADecodeKernel):
 
     @classmethod
     def applies(cls, call: AttentionCall) -> bool:
-        try:
-            native.contiguous_decode_workspace(call.batch, call.q_len, call.heads, call.heads_kv, call.dim,
-                                               max(call.seqlen_kv, 1), call.dtype, call.kv_dtype or call.dtype, 0,
-                                               native.KERNEL_MFMA)
-        except (NotImplementedError, ValueError):
-            return False
-        return True
+        return mfma_kernel_serves(call.dim, 32, call.dtype, call.kv_dtype or call.dtype)  # (walked in 32-token tiles)
 
     @property
     def default_config(self) -> dict[str, Any]:
@@ -494,22 +478,16 @@ class GQAPrefillPagedWithKVCacheFwdKernel(Kernel):
                 v_pages: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
                 cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor, block_table: torch.Tensor, max_seqlen_q: int,
                 cos_table: Optional[torch.Tensor] = None, sin_table: Optional[torch.Tensor] = None) -> torch.Tensor:
-        native.require_gfx950(q.device)
         if cos_table is not None or sin_table is not None:
             raise ValueError(f"{type(self).__name__} takes no rotary tables; the fused-RoPE call is served by "
                              "GQAPrefillPagedWithKVCacheRopeFwdKernel")
         kernel = int(self.config.get("kernel", native.KERNEL_AUTO))
-        nbytes = native.prefill_paged_workspace(self.batch, max_seqlen_q, q.shape[0], self.heads, self.heads_kv, self.dim,
-                                                self.page_size, block_table.shape[1], q.dtype, k_pages.dtype, kernel)
-        out = torch.empty_like(q)
-        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device) if nbytes else None
         if k_scale is None:  # never read with a 16-bit cache; the entry point wants a pointer all the same
             k_scale = v_scale = torch.ones(1, dtype=torch.float32, device=q.device)
-        native.prefill_paged(q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table,
-                             out, workspace, batch=self.batch, max_seqlen_q=max_seqlen_q, heads=self.heads,
-                             heads_kv=self.heads_kv, dim=self.dim, page_size=self.page_size, sm_scale=self.sm_scale,
-                             softcap=self.softcap, causal=self.is_causal, kernel=kernel)
-        return out
+        return torch.ops.tileops_amd.gqa_prefill_paged(
+            q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table, int(max_seqlen_q),
+            self.heads, self.heads_kv, self.dim, self.page_size, float(self.sm_scale), float(self.softcap), bool(self.is_causal),
+            kernel)
 
 
 class GQAPrefillPagedWithFP8KVCacheFwdKernel(GQAPrefillPagedWithKVCacheFwdKernel):
@@ -551,7 +529,6 @@ class GQAPrefillPagedWithKVCacheRopeFwdKernel(GQAPrefillPagedWithKVCacheFwdKerne
                 v_pages: torch.Tensor, k_scale: Optional[torch.Tensor], v_scale: Optional[torch.Tensor],
                 cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor, block_table: torch.Tensor, max_seqlen_q: int,
                 cos_table: Optional[torch.Tensor] = None, sin_table: Optional[torch.Tensor] = None) -> torch.Tensor:
-        native.require_gfx950(q.device)
         if cos_table is None or sin_table is None:
             raise ValueError("the fused-RoPE prefill kernel needs cos_table and sin_table")
         want = (self.max_position, self.rotary_dim // 2)
@@ -560,12 +537,7 @@ class GQAPrefillPagedWithKVCacheRopeFwdKernel(GQAPrefillPagedWithKVCacheFwdKerne
                 raise ValueError(f"{name} must be a contiguous {q.dtype} tensor of shape {want} on {q.device}, got "
                                  f"{t.dtype} {tuple(t.shape)} on {t.device}")
         kernel = int(self.config.get("kernel", native.KERNEL_AUTO))
-        nbytes = native.prefill_paged_rope_workspace(self.batch, max_seqlen_q, q.shape[0], self.heads, self.heads_kv, self.dim,
-                                                     self.page_size, block_table.shape[1], q.dtype, kernel)
-        out = torch.empty_like(q)
-        workspace = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
-        native.prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q, cache_seqlens,
-                                  block_table, out, workspace, batch=self.batch, max_seqlen_q=max_seqlen_q, heads=self.heads,
-                                  heads_kv=self.heads_kv, dim=self.dim, page_size=self.page_size, rotary_dim=self.rotary_dim,
-                                  sm_scale=self.sm_scale, softcap=self.softcap, causal=self.is_causal, kernel=kernel)
-        return out
+        return torch.ops.tileops_amd.gqa_prefill_paged_rope(
+            q, k_new, v_new, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q, cache_seqlens, block_table, int(max_seqlen_q),
+            self.heads, self.heads_kv, self.dim, self.page_size, int(self.rotary_dim), float(self.sm_scale), float(self.softcap),
+            bool(self.is_causal), kernel)

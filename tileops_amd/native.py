@@ -363,6 +363,16 @@ def prefill_input_facts(cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor,
     one transfer to the host."""
     require_gfx950(block_table.device)
     lib = load()
+    # the kernel indexes all three as dense int32 arrays: a direct caller gets an error here, not a wrong fact
+    batch = cache_seqlens.shape[0]
+    if cu_seqlens_q.numel() != batch + 1 or not cu_seqlens_q.is_contiguous() or not cache_seqlens.is_contiguous():
+        raise ValueError(f"cu_seqlens_q must be a contiguous array of {batch + 1} entries and cache_seqlens contiguous, got "
+                         f"{tuple(cu_seqlens_q.shape)} and {tuple(cache_seqlens.shape)}")
+    if any(t.dtype != torch.int32 for t in (cu_seqlens_q, cache_seqlens, block_table)) or block_table.stride(1) != 1:
+        raise ValueError("cu_seqlens_q, cache_seqlens and block_table must be int32, block_table rows contiguous")
+    for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() < 1):
+            raise ValueError(f"{name} must hold at least one float32 value")
     facts = torch.empty(10, dtype=torch.int32, device=block_table.device)
     _check(lib.mi355_prefill_input_facts(
         cu_seqlens_q.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0),

@@ -98,6 +98,9 @@ class Op:
     _overridden_keys: frozenset = frozenset()
     tune: bool = False
     dtype: Optional[torch.dtype] = None
+    #: ``torch.library`` operators this op's call traces to under ``torch.compile(op, fullgraph=True)``
+    #: (reference: ``Op.compile_op_names``, src/tileops/ops/op_base.py:140-147).
+    compile_op_names: tuple = ()
 
     def __init_subclass__(cls, **kwargs: object) -> None:
         super().__init_subclass__(**kwargs)

@@ -78,6 +78,7 @@ class _PagedDecodeOp(Op):
 
     q_len: int = 1
     is_causal: bool = True
+    compile_op_names = ("tileops_amd::gqa_paged_decode",)
     #: Set True to also check values that live on the device (scales finite and positive, block-table
     #: entries inside the pool).  Costs a device read-back per call, so it is off on the serving path.
     debug_checks: bool = False
@@ -93,6 +94,7 @@ class _PagedDecodeOp(Op):
         self.sm_scale = _attention_scale(dim, sm_scale)
         self.softcap = _score_softcap(softcap)
         self.tune = tune
+        self._selected_keys: dict = {}
         if target is not None:
             self.target = target
         self.dispatch_kernel(kernel_map)
@@ -124,7 +126,7 @@ class _PagedDecodeOp(Op):
         # selection is a function of the call and of the kernel map: settled once per (dtypes, device, map), like the
         # reference's once-per-dtype kernel choice (ops/attention/gqa.py:1389-1408)
         memo_key = (dtype, kv_dtype, device, tuple(self.kernel_map.items()))
-        memo = self.__dict__.setdefault("_selected_keys", {})
+        memo = self._selected_keys
         hit = memo.get(memo_key)
         if hit is None:
             call = self.attention_call(dtype, kv_dtype, device)
@@ -298,6 +300,7 @@ class GroupedQueryAttentionDecodeWithKVCacheFwdOp(Op):
     """
 
     _seen_call: Optional[dict] = None
+    compile_op_names = ("tileops_amd::gqa_decode",)
 
     def __init__(self, batch: int, heads: int, heads_kv: int, seqlen_kv: int, dim: int,
                  sm_scale: Optional[float] = None, softcap: Optional[float] = None,
@@ -417,7 +420,12 @@ class GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp(Op):
     reference it reads a few device scalars to do so -- ``validate_inputs=False`` skips exactly those reads).  With ``fuse_rope=True`` (16-bit cache only, as in the reference)
     query and new key rows are rotated at their logical positions before the append; the cos/sin tables are built once
     per (device, dtype) like the reference's (:1048-1065, src/tileops/ops/rope.py:97-120).
+
+    Under ``torch.compile(fullgraph=True)`` the op traces to one operator when built with ``validate_inputs=False``; the
+    value checks read device memory on the host, which no graph can hold (the reference's checks do the same).
     """
+
+    compile_op_names = ("tileops_amd::gqa_prefill_paged", "tileops_amd::gqa_prefill_paged_rope")
 
     def __init__(self, batch: int, heads: int, heads_kv: int, max_pages_per_req: int, page_size: int, dim: int,
                  is_causal: bool = True, cache_dtype: Optional[torch.dtype] = None, sm_scale: Optional[float] = None,

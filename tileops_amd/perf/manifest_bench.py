@@ -12,8 +12,12 @@ Per workload and implementation (tag) it records ``latency_ms`` (median device t
 L2/MALL flushed between calls -- the methodology of benchmarks/timing.py:546-585), ``tflops`` and
 ``bandwidth_tbs`` from the op's ``eval_roofline()`` after it has seen the call, and ``hbm_frac`` = bandwidth over
 the 8 TB/s peak.  ``device_busy_ms`` (sum of kernel durations) is taken from the torch profiler when it delivers
-device events, otherwise left out.  Baseline tag ``torch_sdpa``: ``F.scaled_dot_product_attention`` on the same
-device for the contiguous op (no FlashInfer / AITER build is importable in this image; the tag slot is there).
+device events, otherwise left out.  Baselines on the same device (no FlashInfer / AITER build is importable in this
+image; the tag slot is there): tag ``torch_sdpa`` = ``F.scaled_dot_product_attention`` for the contiguous op; tag
+``torch_gather_sdpa`` = for a paged row, two dense ``index_select`` copies of the pages each sequence addresses followed by
+SDPA with a boolean padding mask and ``enable_gqa`` (torch's math path) -- a plain-torch way to do the same job, not a
+tuned kernel, so its ratio says what a user gains over eager torch and nothing about kernel quality.  Rows with an FP8
+cache, several query tokens or a softcap have no device baseline; the run lists them at its end.
 """
 
 from __future__ import annotations
@@ -250,7 +254,7 @@ def _paged_case(row: dict, dtype: torch.dtype, device: torch.device, multi: bool
 
 def _paged_torch_baseline(op: Any, args: tuple, row: dict, page: int, multi: bool, kv_dtype: torch.dtype) -> Optional[Callable[[], Any]]:
     """torch on the same device for a paged row: gather the pages each sequence addresses into a dense [B, max_len] cache
-    (one ``index_select`` per tensor on an index tensor built from the block table inside the call), then
+    (one ``index_select`` per tensor, on an index tensor built from the block table ahead of the timed call), then
     ``F.scaled_dot_product_attention`` with a padding mask -- the role of the reference benchmark's SDPA baseline
     (benchmarks/ops/attention/bench_gqa_decode_paged.py:21-66) without its per-page host loop.  16-bit caches, one query
     token, no softcap, dense copy of at most 2 GiB; otherwise no baseline."""
@@ -261,15 +265,19 @@ def _paged_torch_baseline(op: Any, args: tuple, row: dict, page: int, multi: boo
         return None
     import torch.nn.functional as F
 
-    def baseline():
-        t = torch.arange(max_len, device=q.device)
-        idx = table.long().gather(1, (t // page).expand(q.shape[0], -1)) * page + t % page  # [B, max_len] physical tokens
-        live = t[None, :] < lens[:, None]
-        idx = torch.where(live, idx, torch.zeros_like(idx))
-        kd = k.index_select(0, idx.reshape(-1)).view(q.shape[0], max_len, k.shape[1], k.shape[2]).transpose(1, 2)
-        vd = v.index_select(0, idx.reshape(-1)).view(q.shape[0], max_len, v.shape[1], v.shape[2]).transpose(1, 2)
-        return F.scaled_dot_product_attention(q.unsqueeze(2), kd, vd, attn_mask=live[:, None, None, :], scale=op.sm_scale, enable_gqa=True)
+    # what depends on the block table and the lengths only is built once, outside the timed call
+    t = torch.arange(max_len, device=q.device)
+    idx = table.long().gather(1, (t // page).expand(q.shape[0], -1)) * page + t % page  # [B, max_len] physical tokens
+    live = t[None, :] < lens[:, None]
+    idx = torch.where(live, idx, torch.zeros_like(idx)).reshape(-1)
+    mask = live[:, None, None, :]
 
+    def baseline():
+        kd = k.index_select(0, idx).view(q.shape[0], max_len, k.shape[1], k.shape[2]).transpose(1, 2)
+        vd = v.index_select(0, idx).view(q.shape[0], max_len, v.shape[1], v.shape[2]).transpose(1, 2)
+        return F.scaled_dot_product_attention(q.unsqueeze(2), kd, vd, attn_mask=mask, scale=op.sm_scale, enable_gqa=True)
+
+    baseline.tag = "torch_gather_sdpa"
     return baseline
 
 
@@ -371,6 +379,7 @@ def main(argv: Optional[list[str]] = None) -> int:
     report, flush = BenchmarkReport(), _Flusher(device)
     suite = ET.Element("testsuite", name="tileops_amd.manifest_bench")
     n = 0
+    no_baseline: list[str] = []
     for op_name, entry in load_manifest().items():
         if op_name not in _CASES or (args.op and args.op != op_name):
             continue
@@ -406,9 +415,12 @@ def main(argv: Optional[list[str]] = None) -> int:
                     bl = _time(baseline, flush, max(args.steps // 2, 3))
                     flops, nbytes = op.eval_roofline()
                     bres = {"latency_ms": bl, "tflops": flops / bl / 1e9, "bandwidth_tbs": nbytes / bl / 1e9}
-                    report.record(op_name, params, bres, "torch_sdpa")
-                    entries.append(dict(bres, tag="torch_sdpa", op=op_name))
-                    line += f"   torch_sdpa {bl * 1e3:9.1f} us (x{bl / lat:.2f})"
+                    tag = getattr(baseline, "tag", "torch_sdpa")
+                    report.record(op_name, params, bres, tag)
+                    entries.append(dict(bres, tag=tag, op=op_name))
+                    line += f"   {tag} {bl * 1e3:9.1f} us (x{bl / lat:.2f})"
+                else:
+                    no_baseline.append(f"{row['label']}-{dname}")
                 junit_case(suite, f"{row['label']}-{dname}", entries)
                 print(line, flush=True)
                 n += 1
@@ -416,6 +428,8 @@ def main(argv: Optional[list[str]] = None) -> int:
                 torch.cuda.empty_cache()
     write_junit(suite, out_dir / "junit.xml")
     report.dump(out_dir / "profile_run.log")
+    if no_baseline:
+        print("no device baseline (FP8 cache, several query tokens, softcap or prefill): " + ", ".join(no_baseline))
     print(f"{n} workloads -> {out_dir}/junit.xml, {out_dir}/profile_run.log")
     return 0
 
