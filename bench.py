@@ -139,6 +139,11 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     per_step_ms, wall = _timed_steps(lambda: op(*args), flush, steps)
     ms = sum(per_step_ms) / steps
     ms_median = statistics.median(per_step_ms)
+    # What the timer reads with nothing between its two records (same flush before): 4-5 us on this stack.  It is NOT a
+    # constant to subtract -- with kernels between the records the pair reads only 1-3 us more than the profiler's sum of
+    # the kernels' durations -- but it is the floor under every event-timed call, and most of a very small call's time.
+    empty_ms, _ = _timed_steps(lambda: None, flush, max(steps, 30))
+    tare_ms = statistics.median(empty_ms)
     # the same K calls back to back (no flush) for reference
     s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s0.record()
@@ -196,7 +201,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     # Device-busy time of a whole call: the sum of the durations of the kernels it launches (attention + merge), launch
     # latency and gaps excluded -- the quantity the reference's own timing protocol reports (its benchmarks take the
     # per-iteration device-busy time from the profiler, benchmarks/timing.py:527-585).  Ten flushed calls.
-    busy = _device_busy_ms(lambda: op(*args), flush, 10)
+    busy = _device_busy_ms(lambda: op(*args), flush, max(steps, 10))
 
     op.observe_call(inp.real_seqlen_kv, cfg.kv_dtype)
     flops, total_bytes = op.eval_roofline()
@@ -237,6 +242,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
             "kv_read_gbs_mean": gbs(kv_read, ms), "kv_read_gbs_median": gbs(kv_read, ms_median),
             "kv_read_frac_of_peak_mean": gbs(kv_read, ms) / HBM_PEAK_GBS, "kv_read_frac_of_peak_median": gbs(kv_read, ms_median) / HBM_PEAK_GBS,
             "all_bytes_frac_of_peak_mean": gbs(total_bytes, ms) / HBM_PEAK_GBS,
+            "event_pair_reads_when_empty_us": tare_ms * 1e3,
         },
         # the attention kernel alone, cold: one launch per HIP-event pair, each after a cache flush (mean of the steps)
         "attention_kernel_us": kernel_ms * 1e3,
@@ -244,7 +250,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
         # the same kernel launched four times back to back per event pair (warm translation and metadata), for reference
         "attention_kernel_us_back_to_back_x4": kernel_b2b_ms * 1e3,
         "frac_back_to_back_x4": total_bytes / (kernel_b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        # dominant kernel alone: algorithmic bytes of one launch / its own cold duration
+        # dominant kernel alone: algorithmic bytes of one launch / its own cold duration (HIP events around the one launch)
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic, "traffic_source": f"{TRAFFIC_SOURCE} (rocprofv3 FETCH_SIZE/WRITE_SIZE of an earlier profiler run, not counted in this run)"},
         "wall_s_timed_region": wall,
@@ -265,7 +271,11 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     if cfg.q_len * (cfg.heads // cfg.heads_kv) >= 16:
         # enough query rows per kv head for the products to be dense matrix work: report the matrix rate beside the bandwidth
         tf = flops / (kernel_ms * 1e-3) / 1e12
-        res["mfma"] = {"flops": flops, "achieved_tflops": tf, "peak_tflops": MFMA_PEAK_TFLOPS, "frac_of_2500": tf / MFMA_PEAK_TFLOPS}
+        from tileops_amd.perf import load_profile
+
+        eff = load_profile("mi355x")["matrix"]["bf16"]["effective_tflops"]  # what a pure matrix-instruction stream sustains (probe)
+        res["mfma"] = {"flops": flops, "achieved_tflops": tf, "peak_tflops": MFMA_PEAK_TFLOPS, "frac_of_2500": tf / MFMA_PEAK_TFLOPS,
+                       "calibrated_peak_tflops": eff, "frac_of_calibrated": tf / eff}
     if with_cpu:
         from oracle.paged_gqa_decode_ref import ref_paged_gqa_decode, ref_paged_gqa_decode_sdpa_math
 

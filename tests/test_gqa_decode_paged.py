@@ -234,6 +234,43 @@ def test_few_sequences_spread_over_hundreds_of_partitions(heads, heads_kv, dim, 
     _run_and_compare(op, case, 64, 3e-2 if fp8 else 2e-2)
 
 
+@pytest.mark.parametrize(
+    "heads, heads_kv, dim, fp8, q_len, lens",
+    [
+        pytest.param(32, 8, 128, False, 1, [4096] + [64] * 15, id="one-sequence-over-a-hundred-partitions-among-short-ones"),
+        pytest.param(32, 8, 128, True, 1, [2048] + [256] * 31, id="fp8-one-sequence-over-dozens-of-partitions"),
+        pytest.param(32, 8, 128, True, 1, [700, 0, 5000, 33, 1, 2000, 64, 900] * 4, id="fp8-ragged-with-empty"),
+        pytest.param(16, 4, 256, False, 1, [3000, 100, 100, 100, 1500, 100, 100, 100] * 2, id="head-dim-256-two-halves"),
+        pytest.param(32, 8, 64, True, 2, [1000 + 37 * i for i in range(32)], id="head-dim-64-fp8-two-query-tokens"),
+        pytest.param(32, 8, 128, False, 1, [20] * 16, id="fewer-tiles-than-partitions-falls-back"),
+    ],
+)
+def test_long_and_short_sequences_share_the_partitions(heads, heads_kv, dim, fp8, q_len, lens):
+    """Batches whose sequences span at most eight partitions on average (the one-wave-per-row merge), with single
+    sequences far outside that average: inside one partition (no merge), over two to eight, over dozens and over more than
+    a hundred partitions (second and later rounds of partial loads), empty ones, and a call with fewer tiles than
+    partitions.  Then a shorter call on the same, now dirty, workspace shapes."""
+    require_gfx950()
+    kv = torch.float8_e4m3fn if fp8 else torch.bfloat16
+    case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, torch.bfloat16, q_len=q_len, fp8=fp8, seed=83)
+    n_parts = native.decode_workspace(len(lens), q_len, heads, heads_kv, dim, 64, case[4].shape[1], torch.bfloat16, kv, 0,
+                                      native.KERNEL_MFMA)[1]
+    assert n_parts <= 8 * len(lens)
+    if q_len == 1:
+        op = PagedOp(len(lens), heads, heads_kv, case[1].shape[0], dim, 64)
+    else:
+        op = MultiOp(len(lens), q_len, heads, heads_kv, case[1].shape[0], dim, 64)
+    _force(op, "gqa_decode_paged_mfma_kernel")
+    tol = 3e-2 if fp8 else 2e-2
+    kw = {"is_causal": True} if q_len > 1 else {}
+    out = _run_and_compare(op, case, 64, tol, **kw)
+    assert out.shape == case[0].shape
+    short = [max(n // 3, 0) for n in lens]
+    case2 = _ragged_case(len(lens), heads, heads_kv, dim, 64, short, torch.bfloat16, q_len=q_len, fp8=fp8, seed=84)
+    if case2[4].shape[1] == case[4].shape[1] and case2[1].shape[0] == case[1].shape[0]:
+        _run_and_compare(op, case2, 64, tol, **kw)
+
+
 def _serves(op, key, dtype, fp8):
     call = op.attention_call(dtype, torch.float8_e4m3fn if fp8 else None, torch.device(DEV, 0))
     return op.kernel_map[key].refusal(call) is None

@@ -358,12 +358,14 @@ def test_chunk_tokens_past_the_block_table_row_are_not_appended(mode):
 
 
 @pytest.mark.gpu
-def test_input_facts_entry_point_against_torch():
+@pytest.mark.parametrize("stride, width", [(512, 300), (511, 301), (512, 3), (513, 513), (2048, 1031)])
+def test_input_facts_entry_point_against_torch(stride, width):
     """mi355_prefill_input_facts on a strided block table with negative entries, a length sum that leaves int32 and a
-    bad scale, against the same reductions in torch."""
+    bad scale, against the same reductions in torch.  Row strides that allow 16-byte loads and ones that do not, widths
+    with and without a tail of fewer than four entries, rows longer than one round of loads."""
     require_gfx950()
     g = torch.Generator().manual_seed(5)
-    batch, width = 37, 300
+    batch = 37
     q_lens = torch.randint(-3, 900, (batch,), generator=g, dtype=torch.int32)
     cu = torch.full((batch + 1,), 7, dtype=torch.int32)
     cu[1:] += torch.cumsum(q_lens, 0).to(torch.int32)
@@ -371,9 +373,10 @@ def test_input_facts_entry_point_against_torch():
     cache[3] = 2**31 - 5  # with any positive q_len the sum leaves int32: the fact saturates
     q_lens[3] = 11
     cu[4:] += 11 - (cu[4] - cu[3])
-    wide = torch.randint(-9, 1 << 22, (batch, 512), generator=g, dtype=torch.int32)
-    table_dev = wide.to(DEV)[:, :width]  # rows 512 entries apart, 300 of them addressed
-    assert not table_dev.is_contiguous()
+    wide = torch.randint(-9, 1 << 22, (batch, stride), generator=g, dtype=torch.int32)
+    wide[:, width:] = torch.randint(-(1 << 30), 1 << 30, (batch, stride - width), generator=g, dtype=torch.int32)  # not addressed: must not count
+    table_dev = wide.to(DEV)[:, :width]  # rows `stride` entries apart, `width` of them addressed
+    assert table_dev.is_contiguous() == (stride == width)
     ks, vs = torch.tensor([0.5], device=DEV), torch.tensor([float("nan")], device=DEV)
     got = native.prefill_input_facts(cu.to(DEV), cache.to(DEV), table_dev, ks, vs)
     ql = (cu[1:] - cu[:-1]).to(torch.int64)
@@ -610,3 +613,56 @@ def test_prefill_kernels_capture_into_a_graph_and_replay_on_new_values(rope):
         assert torch.equal(pages_g[0], k_pages) and torch.equal(pages_g[1], v_pages)
         assert previous is None or not torch.equal(previous, eager)
         previous = eager.clone()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel", [native.KERNEL_GENERIC, native.KERNEL_AUTO], ids=["general", "mfma"])
+@pytest.mark.parametrize("rope", [False, True])
+def test_a_cache_length_near_int_max_is_clamped_not_wrapped(kernel, rope):
+    """With ``validate_inputs=False`` nothing stops a corrupt ``cache_seqlens`` entry.  ``2**31 - 5`` plus an eight-token chunk
+    must not wrap to a negative number (which would read as an empty sequence and return zeros): the length saturates at what
+    the block-table row addresses, the chunk -- whose positions lie outside that row -- is appended nowhere, and the sequence's
+    rows are a bottom-right-causal decode over the row's whole capacity.  The sane sequences of the batch are not disturbed."""
+    require_gfx950()
+    H, Hkv, D, page, max_pages, ql = 32, 8, 128, 64, 4, 8
+    q_lens, old_lens = [ql, ql, ql], [100, 50, 30]
+    case = list(_case(q_lens, old_lens, H, Hkv, D, torch.bfloat16, page=page, max_pages=max_pages, seed=17))
+    g = torch.Generator().manual_seed(18)
+    case[3] = torch.randn(case[3].shape, generator=g).to(torch.bfloat16)  # every pool row holds data: the clamped sequence
+    case[4] = torch.randn(case[4].shape, generator=g).to(torch.bfloat16)  # attends to all 256 tokens of its row
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+    kw = dict(fuse_rope=True, max_position=1024, rotary_dim=D) if rope else {}
+    op = PrefillOp(batch=3, heads=H, heads_kv=Hkv, max_pages_per_req=max_pages, page_size=page, dim=D, is_causal=True,
+                   validate_inputs=False, **kw)
+    dev = [t.to(DEV) for t in case]
+    call = op.attention_call(torch.bfloat16, torch.device(DEV, 0))
+    op._get_kernel(tuple(dev), op.select_kernel_key(tuple(op.kernel_map), call), call).config["kernel"] = kernel
+    bad = cache.clone()
+    bad[1] = 2**31 - 5
+    dev[8] = bad.to(DEV)
+    kp_before, vp_before = dev[3].clone(), dev[4].clone()
+    out = op(*dev, ql).float().cpu()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    kp_after, vp_after = dev[3].cpu(), dev[4].cpu()
+    row1 = torch.cat([torch.arange(int(p) * page, (int(p) + 1) * page) for p in table[1]])
+    assert torch.equal(kp_after[row1], kp_before.cpu()[row1]) and torch.equal(vp_after[row1], vp_before.cpu()[row1])  # nothing appended
+    # the corrupt sequence: a decode of its eight rows over the 256 tokens its table row addresses
+    q1 = q[ql:2 * ql]
+    if rope:
+        cos, sin = op._rope_tables(torch.device(DEV), torch.bfloat16)
+        pos = torch.full((ql,), 1023, dtype=torch.long)  # positions past the tables read the last entry
+        q1 = apply_neox_rope(q1, pos, cos.cpu(), sin.cpu(), D)
+    want1 = ref_paged_gqa_decode(q1.view(1, ql, H, D), kp_after, vp_after, torch.tensor([max_pages * page], dtype=torch.int32), table[1:2],
+                                 page_size=page, is_causal=True).float().view(ql, H, D)
+    torch.testing.assert_close(out[ql:2 * ql], want1, atol=8e-2, rtol=1e-2)
+    assert out[ql:2 * ql].abs().max() > 1e-3  # (zeros are what a wrapped length used to give)
+    # the sane sequences against the oracle run on the uncorrupted lengths
+    if rope:
+        cos, sin = op._rope_tables(torch.device(DEV), torch.bfloat16)
+        ref_out, _, _ = ref_gqa_prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cu, cache, table, cos.cpu(), sin.cpu(),
+                                                   page_size=page, is_causal=True, rotary_dim=D)
+    else:
+        ref_out, _, _ = ref_gqa_prefill_paged(*case, page_size=page, is_causal=True)
+    for b in (0, 2):
+        torch.testing.assert_close(out[b * ql:(b + 1) * ql], ref_out.float()[b * ql:(b + 1) * ql], atol=8e-2, rtol=1e-2)

@@ -100,15 +100,18 @@ const char* launch_kv_append_fp8(const void* x_new, void* cache, float* scale, c
 //   facts[4] cu_q[batch]                             facts[5] max over b of cu_q[b+1] - cu_q[b]
 //   facts[6] min cache_seqlens                       facts[7] max over b of cache_seqlens[b] + q_len[b]   (64-bit sums, saturated)
 //   facts[8] min block_table entry                   facts[9] max block_table entry
-// One workgroup of 256 threads; the block table (batch x max_pages entries, rows bt_row_stride apart) is the long loop.
-__global__ __launch_bounds__(256) void prefill_input_facts_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
-                                                                  const int32_t* __restrict__ block_table, int64_t bt_row_stride,
-                                                                  const float* __restrict__ k_scale, const float* __restrict__ v_scale,
-                                                                  int batch, int max_pages, int32_t* __restrict__ facts) {
-  __shared__ int red[6][256];
-  const int t = threadIdx.x;
+// The block table (batch x max_pages entries, rows bt_row_stride apart) is the bulk of the reading.
+__global__ __launch_bounds__(1024) void prefill_input_facts_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
+                                                                   const int32_t* __restrict__ block_table, int64_t bt_row_stride,
+                                                                   const float* __restrict__ k_scale, const float* __restrict__ v_scale,
+                                                                   int batch, int max_pages, int32_t* __restrict__ facts) {
+  // One workgroup of sixteen waves (the ten facts are global minima and maxima: several workgroups would need a second
+  // launch or initialised memory to meet in).  A wave takes whole block-table rows, 16 bytes per lane and four such loads
+  // in flight when the rows allow it, so that a table of a few thousand entries is one round trip and no index is divided.
+  __shared__ int red[6][16];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   int min_q = INT_MAX, max_q = INT_MIN, min_c = INT_MAX, max_tot = INT_MIN, min_p = INT_MAX, max_p = INT_MIN;
-  for (int b = t; b < batch; b += 256) {
+  for (int b = t; b < batch; b += 1024) {
     const int ql = cu_q[b + 1] - cu_q[b], c = cache_seqlens[b];
     const int64_t tot = (int64_t)c + ql;
     min_q = min(min_q, ql);
@@ -116,44 +119,68 @@ __global__ __launch_bounds__(256) void prefill_input_facts_kernel(const int32_t*
     min_c = min(min_c, c);
     max_tot = max(max_tot, (int)min(max(tot, (int64_t)INT_MIN), (int64_t)INT_MAX));
   }
-  const int64_t n_entries = (int64_t)batch * max_pages;
-  for (int64_t i = t; i < n_entries; i += 256) {
-    const int v = block_table[(i / max_pages) * bt_row_stride + i % max_pages];
-    min_p = min(min_p, v);
-    max_p = max(max_p, v);
-  }
-  red[0][t] = min_q; red[1][t] = max_q; red[2][t] = min_c; red[3][t] = max_tot; red[4][t] = min_p; red[5][t] = max_p;
-  __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if (t < w) {
-      red[0][t] = min(red[0][t], red[0][t + w]);
-      red[1][t] = max(red[1][t], red[1][t + w]);
-      red[2][t] = min(red[2][t], red[2][t + w]);
-      red[3][t] = max(red[3][t], red[3][t + w]);
-      red[4][t] = min(red[4][t], red[4][t + w]);
-      red[5][t] = max(red[5][t], red[5][t + w]);
+  const bool vec_ok = (bt_row_stride & 3) == 0 && ((uintptr_t)block_table & 15) == 0;
+  const int n_vec = vec_ok ? max_pages >> 2 : 0;  // whole 16-byte groups of a row
+  for (int b = wave; b < batch; b += 16) {
+    const int32_t* row = block_table + (int64_t)b * bt_row_stride;
+    for (int j0 = 0; j0 < n_vec; j0 += 256) {
+      int4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int j = j0 + 64 * u + lane;
+        v[u] = ((const int4*)row)[j < n_vec ? j : n_vec - 1];  // (past the end: the last group again)
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        min_p = min(min(min_p, v[u].x), min(v[u].y, min(v[u].z, v[u].w)));
+        max_p = max(max(max_p, v[u].x), max(v[u].y, max(v[u].z, v[u].w)));
+      }
     }
-    __syncthreads();
+    for (int j = 4 * n_vec + lane; j < max_pages; j += 64) {
+      const int v = row[j];
+      min_p = min(min_p, v);
+      max_p = max(max_p, v);
+    }
   }
+  int vals[6] = {min_q, max_q, min_c, max_tot, min_p, max_p};
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+#pragma unroll
+    for (int f = 0; f < 6; f++) {
+      const int o = __shfl_xor(vals[f], m, 64);
+      vals[f] = (f & 1) ? max(vals[f], o) : min(vals[f], o);  // facts 0, 2, 4 are minima, 1, 3, 5 maxima
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int f = 0; f < 6; f++) red[f][wave] = vals[f];
+  }
+  __syncthreads();
   if (t == 0) {
+#pragma unroll
+    for (int f = 0; f < 6; f++) {
+      int r = red[f][0];
+      for (int w = 1; w < 16; w++) r = (f & 1) ? max(r, red[f][w]) : min(r, red[f][w]);
+      vals[f] = r;
+    }
     const float ks = k_scale ? k_scale[0] : 1.f, vs = v_scale ? v_scale[0] : 1.f;
     facts[0] = (isfinite(ks) && ks > 0.f) ? 1 : 0;
     facts[1] = (isfinite(vs) && vs > 0.f) ? 1 : 0;
     facts[2] = cu_q[0];
-    facts[3] = red[0][0];
+    facts[3] = vals[0];
     facts[4] = cu_q[batch];
-    facts[5] = red[1][0];
-    facts[6] = red[2][0];
-    facts[7] = red[3][0];
-    facts[8] = red[4][0];
-    facts[9] = red[5][0];
+    facts[5] = vals[1];
+    facts[6] = vals[2];
+    facts[7] = vals[3];
+    facts[8] = vals[4];
+    facts[9] = vals[5];
   }
 }
 
 const char* launch_prefill_input_facts(const int32_t* cu_q, const int32_t* cache_seqlens, const int32_t* block_table,
                                        int64_t bt_row_stride, const float* k_scale, const float* v_scale, int batch, int max_pages,
                                        int32_t* facts, hipStream_t s) {
-  hipLaunchKernelGGL(prefill_input_facts_kernel, dim3(1), dim3(256), 0, s, cu_q, cache_seqlens, block_table, bt_row_stride, k_scale,
+  hipLaunchKernelGGL(prefill_input_facts_kernel, dim3(1), dim3(1024), 0, s, cu_q, cache_seqlens, block_table, bt_row_stride, k_scale,
                      v_scale, batch, max_pages, facts);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
@@ -178,8 +205,9 @@ __global__ __launch_bounds__(256) void kv_append_chunk_kernel(const uint16_t* __
   }
   const int b = lo;
   if (t >= cu_q[b + 1]) return;
-  const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
-  if (pos < 0 || pos / page_size >= bt_row_stride) return;  // a position the block-table row cannot address: write nothing
+  const int64_t pos64 = (int64_t)cache_seqlens[b] + (t - cu_q[b]);  // (64-bit: a corrupt length near INT_MAX must not wrap)
+  if (pos64 < 0 || pos64 / page_size >= bt_row_stride) return;  // a position the block-table row cannot address: write nothing
+  const int pos = (int)pos64;
   const int64_t phys = physical_token(block_table + (int64_t)b * bt_row_stride, pos, page_size, n_pages);
   const uint16_t* ks = k_new + t * row_elems;
   const uint16_t* vs = v_new + t * row_elems;
@@ -260,9 +288,10 @@ __global__ __launch_bounds__(256) void rope_append_chunk_kernel(const uint16_t* 
   }
   const int b = lo;
   if (t >= cu_q[b + 1]) return;
-  const int pos = cache_seqlens[b] + (int)(t - cu_q[b]);
-  const bool addressable = pos >= 0 && pos / page_size < bt_row_stride;  // else: rotate the query, append nothing
-  const int64_t tpos = pos < max_position ? pos : max_position - 1;  // the caller checks positions; never read past the tables
+  const int64_t pos64 = (int64_t)cache_seqlens[b] + (t - cu_q[b]);  // (64-bit: a corrupt length near INT_MAX must not wrap)
+  const bool addressable = pos64 >= 0 && pos64 / page_size < bt_row_stride;  // else: rotate the query, append nothing
+  const int pos = addressable ? (int)pos64 : 0;
+  const int64_t tpos = pos64 < 0 ? 0 : (pos64 < max_position ? pos64 : max_position - 1);  // the caller checks positions; never read outside the tables
   const int half = rotary_dim >> 1;
   const uint16_t* cs = cos_table + tpos * half;
   const uint16_t* sn = sin_table + tpos * half;
