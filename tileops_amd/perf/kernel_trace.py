@@ -59,14 +59,14 @@ def summary(out_dir: str) -> str:
             stats.setdefault((_short(name), cls), []).append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
             meta[_short(name)] = r
         prev = name
-    lines = ["| kernel | follows | calls | avg us | min us | max us | grid (threads) | workgroup | LDS B | VGPR | AGPR |",
-             "|---|---|---:|---:|---:|---:|---:|---:|---:|---:|---:|"]
+    lines = ["| kernel | follows | calls | avg us | min us | max us | grid (threads) | workgroup | VGPR | AGPR |",
+             "|---|---|---:|---:|---:|---:|---:|---:|---:|---:|"]
     for (name, cls), d in sorted(stats.items()):
         r = meta[name]
         grid = int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
         follows = {"cold": "a cache flush (cold)", "warm": "a kernel of the library (warm)", "other": "another kernel"}[cls]
         lines.append(f"| `{name}` | {follows} | {len(d)} | {statistics.mean(d):.2f} | {min(d):.2f} | {max(d):.2f} | {grid} | "
-                     f"{r['Workgroup_Size_X']} | {r['LDS_Block_Size']} | {r['VGPR_Count']} | {r['Accum_VGPR_Count']} |")
+                     f"{r['Workgroup_Size_X']} | {r['VGPR_Count']} | {r['Accum_VGPR_Count']} |")
     return "\n".join(lines)
 
 
