@@ -53,6 +53,12 @@ constexpr int kD = 128;       // default head dim (64 and 256 also run)
 // Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
 constexpr bool kLateIssueNarrow = true;
+// Shared rings of four stages consume two tiles per barrier where two tiles of one sequence are left: one wait, one
+// barrier and one round of fetch requests per 64 tokens instead of per 32.
+#ifndef MI355_PAIR_STEPS
+#define MI355_PAIR_STEPS 1
+#endif
+constexpr bool kPairSteps = MI355_PAIR_STEPS != 0;
 
 // Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
 // hold row groups past the last query row, which load nothing, mask everything and store nothing.
@@ -1064,13 +1070,39 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     }
   };
   int u = 0, ring = 0, seg_count = 0;
+  // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
+  constexpr bool RESCALE_IN_LOOP = (SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2);
+  constexpr bool PAIRS = kPairSteps && SH && NS >= 4 && D <= 128 && RESCALE_IN_LOOP;
+  constexpr int STEP = PAIRS ? NS / 2 : 1;  // tiles per barrier: half the ring is read while the other half is refilled
   while (u < n_units) {
     const int seg_first_j = cc.j;
     const int seg_units = min(cc.nt - cc.j, n_units - u);
     if (!LATE) issue_ahead(ring);  // before the query loads, so the next tile is already in flight while they land
     begin_segment(cc);
     int k = 0;
-    while (k < seg_units) {
+    if constexpr (PAIRS) {
+      while (k < seg_units) {
+        const int step = min(STEP, seg_units - k);  // tiles of this step: u .. u + step - 1, in ring slots u % NS and on
+        wait_stage(u + step - 1);                    // the later tile has landed, so has the earlier (requests complete in order)
+        // Past the barrier every wave's part of both tiles is in LDS, and every wave has finished reading the tiles before
+        // u: their slots may be refilled.  Tile t goes to slot t % NS, so the request may run up to tile u + NS - 1.
+        asm volatile("s_barrier" ::: "memory");
+        while (issued < n_units && issued - NS < u) {
+          issue(ci, issued & (NS - 1), ci_row);
+          if (++issued < n_units) advance();
+        }
+#pragma nounroll
+        for (int sub = 0; sub < step; ++sub) {  // (a loop, not two copies: the body is large)
+          if (__builtin_expect(run_score_step(ring), 0)) rescale();
+          value_step((uint32_t)ring * G::STAGE);
+          ++u;
+          ++cc.j;
+          ring = (ring + 1) & (NS - 1);
+          ++k;
+        }
+      }
+    }
+    while (!PAIRS && k < seg_units) {
       bool moved = false;
       for (; k < seg_units; ++k) {  // steady state: no tile in here rescales the accumulators
         if (!LATE && k > 0) issue_ahead(ring);
@@ -1082,8 +1114,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
         }
         if (LATE) issue_ahead(ring);
         moved = run_score_step(ring);
-        if constexpr ((SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2)) {
-          // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
+        if constexpr (RESCALE_IN_LOOP) {
           if (__builtin_expect(moved, 0)) rescale();
           moved = false;
         } else {
@@ -1551,7 +1582,10 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
       if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of four waves for this row width";
     default:
-      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+#ifndef MI355_RING8_STAGES
+#define MI355_RING8_STAGES 4
+#endif
+      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, (D == 128 && !Geom<KVT, D>::FP8) ? MI355_RING8_STAGES : 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
