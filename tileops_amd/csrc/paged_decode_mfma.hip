@@ -54,11 +54,8 @@ constexpr int kD = 128;       // default head dim (64 and 256 also run)
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
 constexpr bool kLateIssueNarrow = true;
 // Shared rings of four stages consume two tiles per barrier where two tiles of one sequence are left: one wait, one
-// barrier and one round of fetch requests per 64 tokens instead of per 32.
-#ifndef MI355_PAIR_STEPS
-#define MI355_PAIR_STEPS 1
-#endif
-constexpr bool kPairSteps = MI355_PAIR_STEPS != 0;
+// barrier and one round of fetch requests per 64 tokens instead of per 32 (head dims up to 128; at 256 it measured 6 % slower).
+constexpr bool kPairSteps = true;
 
 // Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
 // hold row groups past the last query row, which load nothing, mask everything and store nothing.
@@ -1582,10 +1579,8 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
       if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of four waves for this row width";
     default:
-#ifndef MI355_RING8_STAGES
-#define MI355_RING8_STAGES 4
-#endif
-      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, (D == 128 && !Geom<KVT, D>::FP8) ? MI355_RING8_STAGES : 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      // (four stages: a ring of eight stages read four tiles per barrier measured 1.5 % faster at twice the LDS -- not taken)
+      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
