@@ -387,6 +387,41 @@ def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, 
         torch.testing.assert_close(out.float(), ref2.float(), atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("num_split", [1, 2, 3, 7])
+@pytest.mark.parametrize(
+    "q_len, heads, heads_kv, dim, fp8",
+    [
+        pytest.param(8, 64, 8, 128, True, id="fp8-ring-of-2"),
+        pytest.param(16, 32, 4, 128, True, id="fp8-ring-of-4"),
+        pytest.param(16, 32, 4, 128, False, id="bf16-ring-of-4"),
+        pytest.param(32, 32, 4, 128, False, id="bf16-ring-of-8"),
+        pytest.param(8, 64, 8, 64, False, id="bf16-head-dim-64-ring-of-2"),
+        pytest.param(32, 32, 4, 256, False, id="bf16-head-dim-256-ring-of-8-one-tile-per-barrier"),
+    ],
+)
+def test_ring_waves_walk_many_tiles_over_sequence_borders(num_split, q_len, heads, heads_kv, dim, fp8):
+    """The tile stream cut into one, two, three or seven ranges only, so that every wave of a shared ring walks dozens
+    of tiles: steps of two tiles per barrier (half of a four-stage ring) wherever two tiles of one sequence are left,
+    steps of one at the end of sequences with an odd number of tiles, at one-tile sequences and at the end of a range,
+    with the ring's refill running across sequence borders.  Against the oracle, NaN in every unaddressed token."""
+    require_gfx950()
+    lens = [2100, q_len, q_len + 33, 700, 64 + q_len, q_len + 1, 1500, 96, 4000]
+    case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, torch.bfloat16, q_len=q_len, fp8=fp8, seed=97)
+    q, k, v, seqlens, table, ks, vs = case
+    ref = ref_paged_gqa_decode(q, k, v, seqlens, table, page_size=64, k_scale=ks, v_scale=vs, is_causal=True)
+    dev = [None if t is None else t.to(DEV) for t in case]
+    out = torch.ops.tileops_amd.gqa_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], q_len, heads, heads_kv, dim, 64,
+                                                 dim ** -0.5, 0.0, True, num_split, native.KERNEL_MFMA)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    tol = 3e-2 if fp8 else 2e-2
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=tol, rtol=tol)
+    # the same call cut into the default number of ranges (a tile or two per wave) differs by fp32 summation order only
+    auto = torch.ops.tileops_amd.gqa_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], q_len, heads, heads_kv, dim, 64,
+                                                  dim ** -0.5, 0.0, True, 0, native.KERNEL_MFMA)
+    torch.testing.assert_close(out.float(), auto.float(), atol=tol, rtol=tol)
+
+
 @pytest.mark.parametrize("softcap", [0.0, 30.0])
 def test_closed_forms_on_device(softcap):
     require_gfx950()
