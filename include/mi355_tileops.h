@@ -249,8 +249,9 @@ int mi355_kv_append_fp8(const void* x_new, void* cache, float* scale, const int3
 /*
  * The facts behind the value checks that the reference's paged prefill op makes on the host before it launches
  * (GroupedQueryAttentionPrefillPagedWithKVCacheFwdOp._validate_forward_inputs, src/tileops/ops/attention/gqa.py:997-1040:
- * each there a device-to-host read of its own), reduced by one small kernel into ten int32 in device memory so that a
- * caller reads them in one transfer:
+ * each there a device-to-host read of its own), reduced by one small kernel into ten int32 so that a caller reads them
+ * in one transfer (facts: device memory, or pinned host memory, which the kernel writes directly and the caller reads after
+ * waiting for the stream):
  *   facts[0], facts[1]  k_scale[0], v_scale[0] finite and positive (1/0; a null scale pointer counts as good)
  *   facts[2] cu_seqlens_q[0]           facts[3] min q_len     facts[4] cu_seqlens_q[batch]   facts[5] max q_len
  *   facts[6] min cache_seqlens         facts[7] max (cache_seqlens + q_len), saturated to int32

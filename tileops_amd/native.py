@@ -46,6 +46,7 @@ class NativeLibraryError(RuntimeError):
 
 _lock = threading.Lock()
 _lib: Optional[ctypes.CDLL] = None
+_facts_local = threading.local()  # per-thread pinned buffer of prefill_input_facts
 
 _c_int, _c_i64, _c_f32, _c_vp, _c_sz = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 
@@ -373,9 +374,16 @@ def prefill_input_facts(cu_seqlens_q: torch.Tensor, cache_seqlens: torch.Tensor,
     for name, t in (("k_scale", k_scale), ("v_scale", v_scale)):
         if t is not None and (t.dtype != torch.float32 or t.numel() < 1):
             raise ValueError(f"{name} must hold at least one float32 value")
-    facts = torch.empty(10, dtype=torch.int32, device=block_table.device)
+    # The kernel writes the ten values straight into pinned host memory (device-addressable at the same address), and the
+    # host waits for the stream: no device buffer, no copy back.  One buffer per thread, so that threads that drive
+    # different streams do not share it.
+    facts = getattr(_facts_local, "buf", None)
+    if facts is None:
+        facts = _facts_local.buf = torch.empty(10, dtype=torch.int32, pin_memory=True)
+    stream = torch.cuda.current_stream(block_table.device)
     _check(lib.mi355_prefill_input_facts(
         cu_seqlens_q.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         k_scale.data_ptr() if k_scale is not None else None, v_scale.data_ptr() if v_scale is not None else None,
-        cache_seqlens.shape[0], block_table.shape[1], facts.data_ptr(), _stream_ptr(block_table.device)))
+        cache_seqlens.shape[0], block_table.shape[1], facts.data_ptr(), stream.cuda_stream))
+    stream.synchronize()
     return facts.tolist()
