@@ -7,7 +7,7 @@
 //
 //  * Work unit = one wave.  A wave owns (partition, kv head, block of query rows) and runs on its own; only when a
 //    kv head has several blocks of query rows do 2, 4 or 8 such waves share their LDS stages and meet at one
-//    barrier per tile (see the kernel's template parameter SHW).  The KV "tile stream" (every 32-token tile of
+//    barrier per tile, or per two tiles on rings of four stages (see the kernel's template parameter SHW).  The KV "tile stream" (every 32-token tile of
 //    every sequence, in batch order) is cut into n_parts equal contiguous ranges computed on the device from
 //    real_seqlen_kv, so all
 //    compute units get the same number of tiles whatever the length distribution, and nothing is read back
@@ -251,8 +251,9 @@ __device__ __forceinline__ void cursor_next(Cursor& c, const DecodeParams& p, bo
 // ------------------------------------------------------------------------------------------------------
 // SHW > 1 (shared stages): when the row groups of a kv head come in multiples of SHW, a workgroup is SHW waves that
 // serve SHW consecutive row groups of the same (partition, kv head), i.e. they walk the same tiles.  They share one
-// LDS ring: each fetches 1/SHW of every stage, and one barrier per tile makes all parts visible and retires the slot
-// that is refilled next.  All waves execute the same number of barriers because they own the same tile range.
+// LDS ring: each fetches 1/SHW of every stage, and one barrier per step (one tile, or two on a ring of four stages at
+// head dims up to 128) makes all parts visible and retires the slots that are refilled next.  All waves execute the same
+// number of barriers because they own the same tile range.
 template <typename QT, typename KVT, int NRB, int NS, int NW, int SHW, int D>
 __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 1) void paged_decode_mfma_kernel(const DecodeParams p, int* __restrict__ ws_prefix) {
   using G = Geom<KVT, D>;
