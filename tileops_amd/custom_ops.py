@@ -32,6 +32,7 @@ OP_NAMES = ("tileops_amd::gqa_paged_decode", "tileops_amd::gqa_decode", "tileops
 # (workspace bytes, partition count) per shape: a workspace query touches no device and never changes its answer
 _decode_plans: dict[tuple, tuple[int, int]] = {}
 _contig_plans: dict[tuple, tuple[int, int]] = {}
+_prefill_plans: dict[tuple, int] = {}
 
 
 def _workspace(nbytes: int, device: torch.device) -> Optional[torch.Tensor]:
@@ -98,8 +99,11 @@ def gqa_prefill_paged(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
     """Packed prefill chunk with paged-cache append (``mi355_gqa_prefill_paged``); writes the chunk into the pages."""
     native.require_gfx950(q.device)
     batch = cache_seqlens.shape[0]
-    nbytes = native.prefill_paged_workspace(batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, block_table.shape[1],
-                                            q.dtype, k_pages.dtype, kernel)
+    key = (batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, block_table.shape[1], q.dtype, k_pages.dtype, kernel)
+    nbytes = _prefill_plans.get(key)
+    if nbytes is None:
+        nbytes = _prefill_plans[key] = native.prefill_paged_workspace(batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size,
+                                                                      block_table.shape[1], q.dtype, k_pages.dtype, kernel)
     out = torch.empty_like(q)
     native.prefill_paged(q, k_new, v_new, k_pages, v_pages, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table, out,
                          _workspace(nbytes, q.device), batch=batch, max_seqlen_q=max_seqlen_q, heads=heads, heads_kv=heads_kv, dim=dim,
@@ -121,8 +125,11 @@ def gqa_prefill_paged_rope(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Te
     """The same with rotary position embedding fused in (``mi355_gqa_prefill_paged_rope``)."""
     native.require_gfx950(q.device)
     batch = cache_seqlens.shape[0]
-    nbytes = native.prefill_paged_rope_workspace(batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size,
-                                                 block_table.shape[1], q.dtype, kernel)
+    key = (batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim, page_size, block_table.shape[1], q.dtype, "rope", kernel)
+    nbytes = _prefill_plans.get(key)
+    if nbytes is None:
+        nbytes = _prefill_plans[key] = native.prefill_paged_rope_workspace(batch, max_seqlen_q, q.shape[0], heads, heads_kv, dim,
+                                                                           page_size, block_table.shape[1], q.dtype, kernel)
     out = torch.empty_like(q)
     workspace = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
     native.prefill_paged_rope(q, k_new, v_new, k_pages, v_pages, cos_table, sin_table, cu_seqlens_q, cache_seqlens, block_table, out,

@@ -25,6 +25,7 @@ from __future__ import annotations
 import argparse
 import statistics
 import sys
+import time
 import xml.etree.ElementTree as ET
 from datetime import datetime
 from pathlib import Path
@@ -184,8 +185,25 @@ class _Flusher:
         self.r.max()
 
 
-def _time(fn: Callable[[], Any], flush: _Flusher, steps: int, warmup: int = 3) -> float:
-    for _ in range(warmup):
+#: warm-up budget and iteration clamp of the reference's protocol (benchmarks/timing.py:30-36, :577): as many untimed,
+#: flushed iterations as fit 25 ms, at least 10 and at most 200.  After idle the device runs its first tens of
+#: milliseconds below its sustained clocks (the 8 x 512-token prefill row reads 465 us in its first twenty calls and
+#: 427 us from the fortieth on), so a row timed after three warm-up calls reports the ramp, not the kernel.
+_DRY_RUN_MS, _MIN_ITERS, _MAX_ITERS = 25.0, 10, 200
+
+
+def _time(fn: Callable[[], Any], flush: _Flusher, steps: int) -> float:
+    flush()
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):  # calibration: one flushed iteration costs this much
+        flush()
+        fn()
+    torch.cuda.synchronize()
+    per_iter_ms = max((time.perf_counter() - t0) * 1e3 / 3, 1e-3)
+    for _ in range(min(max(int(_DRY_RUN_MS / per_iter_ms), _MIN_ITERS), _MAX_ITERS)):
+        flush()
         fn()
     ts = []
     for _ in range(steps):
