@@ -180,8 +180,12 @@ int mi355_gqa_decode(const void* q, const void* k, const void* v, const float* k
  *   out            [total_q, heads, dim] q_dtype
  *   max_seqlen_q   upper bound of the chunk lengths (sizes the launch; a longer chunk would lose its last rows)
  *   causal         query i of a chunk sees the old tokens and chunk tokens j <= i (gqa_fwd.py:1247-1256); 0: all of them
- * Attention runs over the dequantised old tokens and the *unquantised* chunk (as the reference: :1180-1245): with an fp8
- * cache that is two passes (pages, then k_new/v_new) whose fp32 results are merged by log-sum-exp.
+ * Attention runs over the dequantised old tokens and the *unquantised* chunk (as the reference: :1180-1245).  With an fp8
+ * cache that is either two passes (the fp8 pages, then k_new/v_new, merged by log-sum-exp) or, from 1024 query rows per
+ * kv head (max_seqlen_q * heads / heads_kv) on the MFMA kernel, one pass over rows dequantised once into the workspace
+ * as (fp8 * scale) rounded to q_dtype (the reference's own dequantisation, :1063-1065) with the chunk behind them.  The
+ * second form needs 4 * batch * max_pages_per_req * page_size * heads_kv * dim bytes of workspace and is only taken up
+ * to 4 GiB of it; the workspace query answers for whichever form the same arguments select.
  * Sequences with an empty chunk produce no output rows and append nothing.  A chunk token whose position
  * cache_seqlens[b] + i the block-table row cannot address (negative, or page index >= bt_row_stride) is not appended.
  */

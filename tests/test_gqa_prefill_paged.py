@@ -439,6 +439,40 @@ def test_llama_shape_chunks_of_hundreds_of_rows_against_long_prefixes(fp8):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("is_causal", [True, False])
+def test_fp8_cache_long_chunks_make_one_pass_over_rows_dequantised_once_and_wide_tables_keep_two_passes(dtype, is_causal):
+    """From 1024 query rows per kv head an FP8-cache call dequantises the cached tokens once into contiguous 16-bit rows
+    (as the reference does: ``(fp8.float() * scale).to(dtype)``), copies the chunk behind them and makes one 16-bit pass;
+    the workspace query says so.  The same call through a block table as wide as a large pool would need more workspace than
+    the library takes for this, keeps the two passes (fp8 pages, then the chunk), and agrees.  Chunks of 300, 256 and 1
+    tokens at group 4, an empty cache, a chunk that ends mid-page."""
+    require_gfx950()
+    q_lens, old_lens, heads, heads_kv, dim, page, max_pages = [300, 256, 1], [1000, 0, 77], 16, 4, 128, 64, 24
+    case = _case(q_lens, old_lens, heads, heads_kv, dim, dtype, fp8=True, page=page, max_pages=max_pages, seed=41)
+    packed_rows = len(q_lens) * max_pages * page * heads_kv * dim * 2 * 2
+    narrow = native.prefill_paged_workspace(len(q_lens), max(q_lens), sum(q_lens), heads, heads_kv, dim, page, max_pages, dtype, FP8,
+                                            native.KERNEL_AUTO)
+    assert narrow >= packed_rows
+    op = PrefillOp(batch=len(q_lens), heads=heads, heads_kv=heads_kv, max_pages_per_req=max_pages, page_size=page, dim=dim,
+                   cache_dtype=FP8, is_causal=is_causal)
+    out = _run(op, case, page, dtype, fp8=True, causal=is_causal)
+    wide_pages = 600_000
+    wide = native.prefill_paged_workspace(len(q_lens), max(q_lens), sum(q_lens), heads, heads_kv, dim, page, wide_pages, dtype, FP8,
+                                          native.KERNEL_AUTO)
+    wider = native.prefill_paged_workspace(len(q_lens), max(q_lens), sum(q_lens), heads, heads_kv, dim, page, wide_pages + 100_000, dtype,
+                                           FP8, native.KERNEL_AUTO)
+    assert wide == wider  # no packed rows in it: it does not grow with the table
+    table = torch.zeros(len(q_lens), wide_pages, dtype=torch.int32)
+    table[:, :max_pages] = case[9]
+    case_wide = (*case[:9], table)
+    op_wide = PrefillOp(batch=len(q_lens), heads=heads, heads_kv=heads_kv, max_pages_per_req=wide_pages, page_size=page, dim=dim,
+                        cache_dtype=FP8, is_causal=is_causal)
+    out_wide = _run(op_wide, case_wide, page, dtype, fp8=True, causal=is_causal)
+    torch.testing.assert_close(out.float(), out_wide.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dim, heads, heads_kv", [(256, 16, 4), (64, 16, 2), (256, 8, 8)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_head_dims_64_and_256_with_chunks_of_hundreds_of_rows(dim, heads, heads_kv, dtype):

@@ -402,12 +402,58 @@ static int prefill_plans(int batch, int max_seqlen_q, int heads, int heads_kv, i
   return rc;
 }
 
+// FP8 cache with long chunks: instead of one pass over the fp8 pages and one over the chunk, the cached tokens are
+// dequantised once into contiguous 16-bit rows (dequant_pack_chunk_kernel), the chunk's tokens copied behind them, and the
+// 16-bit kernel makes one pass over both.  Converting in the attention kernel costs every wave that reads a tile its own
+// conversion (8 x 512-token chunks on 4 K prefixes: 448 us + 80 us for the chunk against 405 us for the one 16-bit pass);
+// converting once costs the cache's bytes five times over (read 1, write 2, read 2), which only pays while the attention
+// is compute-bound: from kPackMinRows query rows per kv head, on the MFMA kernel, within kPackMaxBytes of workspace
+// (a block table as wide as the whole pool asks for more and keeps the two passes).
+constexpr int kPackMinRows = 1024;
+constexpr size_t kPackMaxBytes = (size_t)4 << 30;
+struct PackPlan {
+  bool use = false;
+  int stride = 0;          // token rows per sequence slot
+  size_t starts_bytes = 0; // kv_starts[batch]
+  size_t kv_bytes = 0;     // one of the two packed tensors
+  Plan attn;               // the single 16-bit pass
+};
+
+static int fp8_prefill_pack_plan(int batch, int max_seqlen_q, int heads, int heads_kv, int dim, int page_size,
+                                 int64_t max_pages_per_req, int q_dtype, int kernel, PackPlan* pp) {
+  *pp = PackPlan();
+  if ((kernel & 0xFF) == MI355_KERNEL_GENERIC) return MI355_OK;
+  if ((int64_t)max_seqlen_q * (heads / heads_kv) < kPackMinRows) return MI355_OK;
+  const int64_t stride = (max_pages_per_req * page_size + kContigTile - 1) / kContigTile * kContigTile;
+  if (stride <= 0 || stride * batch >= INT_MAX) return MI355_OK;
+  const size_t kv_bytes = align256((size_t)batch * stride * heads_kv * dim * 2);
+  if (2 * kv_bytes > kPackMaxBytes) return MI355_OK;
+  int rc = make_plan(batch, max_seqlen_q, heads, heads_kv, dim, kContigTile, stride / kContigTile, q_dtype, q_dtype, 0.f, 0, kernel,
+                     &pp->attn);
+  if (rc) return rc;
+  if (pp->attn.kernel != MI355_KERNEL_MFMA) return MI355_OK;
+  pp->use = true;
+  pp->stride = (int)stride;
+  pp->starts_bytes = align256((size_t)batch * sizeof(int32_t));
+  pp->kv_bytes = kv_bytes;
+  return MI355_OK;
+}
+
 int mi355_gqa_prefill_paged_workspace(int batch, int max_seqlen_q, int64_t total_q, int heads, int heads_kv, int dim,
                                       int page_size, int64_t max_pages_per_req, int q_dtype, int cache_dtype, int kernel,
                                       size_t* workspace_bytes) {
   int rc = check_shape(batch, max_seqlen_q, heads, heads_kv, dim, page_size, q_dtype, cache_dtype);
   if (rc) return rc;
   if (total_q < 0) return fail(MI355_EINVAL, "total_q must be non-negative");
+  if (cache_dtype == MI355_DT_FP8_E4M3FN) {
+    PackPlan pp;
+    rc = fp8_prefill_pack_plan(batch, max_seqlen_q, heads, heads_kv, dim, page_size, max_pages_per_req, q_dtype, kernel, &pp);
+    if (rc) return rc;
+    if (pp.use) {
+      if (workspace_bytes) *workspace_bytes = align256(pp.attn.part_o_bytes + pp.attn.part_lse_bytes) + pp.starts_bytes + 2 * pp.kv_bytes;
+      return MI355_OK;
+    }
+  }
   Plan a, b;
   rc = prefill_plans(batch, max_seqlen_q, heads, heads_kv, dim, page_size, max_pages_per_req, q_dtype, cache_dtype, kernel, &a, &b);
   if (rc) return rc;
@@ -455,6 +501,26 @@ int mi355_gqa_prefill_paged(const void* q, const void* k_new, const void* v_new,
   if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
   Extras ex;
   ex.cu_q = cu_seqlens_q;
+  if (fp8) {
+    PackPlan pp;
+    rc = fp8_prefill_pack_plan(batch, max_seqlen_q, heads, heads_kv, dim, page_size, bt_row_stride, q_dtype, kernel, &pp);
+    if (rc) return rc;
+    if (pp.use) {
+      const size_t attn_bytes = align256(pp.attn.part_o_bytes + pp.attn.part_lse_bytes);
+      int32_t* starts = (int32_t*)((char*)workspace + attn_bytes);
+      void* kp = (char*)workspace + attn_bytes + pp.starts_bytes;
+      void* vp = (char*)kp + pp.kv_bytes;
+      err = launch_dequant_pack_chunk(k_pages, v_pages, k_new, v_new, k_scale, v_scale, cu_seqlens_q, cache_seqlens, block_table,
+                                      bt_row_stride, kp, vp, starts, batch, heads_kv, dim, page_size, n_phys_tokens / page_size,
+                                      pp.stride, q_dtype, s);
+      if (err) return fail(MI355_ELAUNCH, "kernel launch failed: %s", err);
+      ex.len_excludes_new = 1;
+      ex.kv_starts = starts;
+      return run_decode(q, kp, vp, nullptr, nullptr, cache_seqlens, nullptr, pp.stride / kContigTile, 0, 0, out, workspace, attn_bytes,
+                        batch, max_seqlen_q, heads, heads_kv, dim, kContigTile, (int64_t)batch * pp.stride, q_dtype, q_dtype, sm_scale,
+                        softcap, causal, 0, kernel, hip_stream, ex);
+    }
+  }
   if (!fp8) {
     // 16-bit cache: the chunk is in the pages now, bit for bit; one pass over (old + new) tokens
     ex.len_excludes_new = 1;

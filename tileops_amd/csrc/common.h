@@ -140,6 +140,11 @@ const char* launch_rope_append_chunk(const void* q, const void* k_new, const voi
                                      const int32_t* cache_seqlens, const int32_t* block_table, int64_t bt_row_stride, int batch,
                                      int64_t total_q, int heads, int heads_kv, int dim, int rotary_dim, int64_t max_position,
                                      int page_size, int64_t n_pages, int x_dtype, hipStream_t s);
+const char* launch_dequant_pack_chunk(const void* k_pages, const void* v_pages, const void* k_new, const void* v_new,
+                                      const float* k_scale, const float* v_scale, const int32_t* cu_q, const int32_t* cache_seqlens,
+                                      const int32_t* block_table, int64_t bt_row_stride, void* kp, void* vp, int32_t* kv_starts,
+                                      int batch, int heads_kv, int dim, int page_size, int64_t n_pages, int stride, int x_dtype,
+                                      hipStream_t s);
 const char* launch_merge_two(const float* o_a, const float* lse_a, const float* o_b, const float* lse_b, void* out,
                              int64_t rows, int dim, int q_dtype, hipStream_t s);
 const char* launch_prefill_input_facts(const int32_t* cu_q, const int32_t* cache_seqlens, const int32_t* block_table,

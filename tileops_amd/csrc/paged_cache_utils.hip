@@ -378,6 +378,113 @@ const char* launch_rope_append_chunk(const void* q, const void* k_new, const voi
   return e == hipSuccess ? nullptr : hipGetErrorString(e);
 }
 
+// FP8 cache, prefill chunk: every sequence's keys (and values) as one contiguous run of 16-bit rows -- the cached tokens
+// gathered through the block table and dequantised as the reference does, (fp8.float() * scale).to(dtype) with one scale
+// per tensor (gqa_fwd.py:1063-1065), followed by the chunk's own tokens as they came.  Sequence b occupies rows
+// [b*stride, b*stride + len_b) of kp / vp, len_b = the length the attention kernel will form from the same two arrays
+// (seq_len_finish: cache length + chunk length, clamped to the slot); kv_starts[b] = b*stride is written here too.
+// One pass of the 16-bit attention kernel over these rows then replaces a pass over the fp8 pages plus a pass over
+// the chunk: the bytes are converted once per call instead of once per wave that reads them.
+// grid (ceil(stride / 64), batch): a workgroup packs 64 token rows, eight elements (16 bytes of output) per thread.
+template <typename XT>
+__global__ __launch_bounds__(256) void dequant_pack_chunk_kernel(const uint8_t* __restrict__ k_pages, const uint8_t* __restrict__ v_pages,
+                                                                 const uint16_t* __restrict__ k_new, const uint16_t* __restrict__ v_new,
+                                                                 const float* __restrict__ k_scale, const float* __restrict__ v_scale,
+                                                                 const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cache_seqlens,
+                                                                 const int32_t* __restrict__ block_table, int64_t bt_row_stride,
+                                                                 uint16_t* __restrict__ kp, uint16_t* __restrict__ vp,
+                                                                 int32_t* __restrict__ kv_starts, int64_t row_elems, int page_size,
+                                                                 int64_t n_pages, int stride, int table_tokens, int tpt_shift) {
+  const int b = blockIdx.y;
+  if (blockIdx.x == 0 && threadIdx.x == 0) kv_starts[b] = b * stride;
+  const int q0 = cu_q[b], ql = cu_q[b + 1] - q0;
+  if (ql <= 0) return;  // no query rows: the attention kernel gives this sequence no tile
+  int cached = cache_seqlens[b];
+  cached = cached < 0 ? 0 : cached;
+  const int len = cached > stride - ql ? stride : cached + ql;  // == seq_len_finish() with max_len = stride
+  const int n_old = min(min(cached, len), table_tokens);        // (a corrupt length cannot run the gather past the table row)
+  const int t_end = min(len, (int)(blockIdx.x + 1) * 64);
+  const float sk = k_scale[0], sv = v_scale[0];
+  const int32_t* bt_row = block_table + (int64_t)b * bt_row_stride;
+  // tpt threads per token row (the power of two that covers row_elems / 8, at most 256), 256 / tpt rows per round.
+  // Eight rounds at a time, every load of the eight issued before the first is used and none behind a branch (a row that is
+  // not of the kind a load is for reads a clamped neighbour and drops it): the kernel moves a few bytes per thread per
+  // round, so what it needs is loads in flight, not arithmetic.
+  const int sub = threadIdx.x >> tpt_shift, lane_e = threadIdx.x & ((1 << tpt_shift) - 1), rows_per_round = 256 >> tpt_shift;
+  const int per_row = (int)(row_elems / 8);
+  constexpr int UN = 8;
+  const int last_old = max(n_old - 1, 0);
+  // pages of a multiple of 64 tokens: the workgroup's 64 tokens lie in one page, one table entry serves them all
+  const bool one_page = (page_size & 63) == 0;
+  const int blk0 = (int)blockIdx.x * 64;
+  const int64_t phys_blk = physical_token(bt_row, min(blk0, last_old), page_size, n_pages) - min(blk0, last_old);
+  for (int c = lane_e; c < per_row; c += 1 << tpt_shift) {  // (one trip unless a row is wider than 256 threads x 8 elements)
+    const int64_t e = (int64_t)c * 8;
+    for (int t0 = (int)blockIdx.x * 64 + sub; t0 < t_end; t0 += UN * rows_per_round) {
+      int64_t phys[UN];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int tc = min(t0 + u * rows_per_round, last_old);
+        phys[u] = one_page ? phys_blk + tc : physical_token(bt_row, tc, page_size, n_pages);
+      }
+      u32x2 kr[UN], vr[UN];
+      uint4 kn[UN], vn[UN];
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int t = t0 + u * rows_per_round;
+        const int64_t src_old = phys[u] * row_elems + e;
+        const int64_t src_new = ((int64_t)q0 + min(max(t - cached, 0), ql - 1)) * row_elems + e;  // chunk token t - cached
+        kr[u] = *(const u32x2*)(k_pages + src_old);
+        vr[u] = *(const u32x2*)(v_pages + src_old);
+        kn[u] = *(const uint4*)(k_new + src_new);
+        vn[u] = *(const uint4*)(v_new + src_new);
+      }
+#pragma unroll
+      for (int u = 0; u < UN; u++) {
+        const int t = t0 + u * rows_per_round;
+        if (t >= t_end) continue;
+        if (t < n_old) {
+          const uint32_t kw[2] = {kr[u][0], kr[u][1]}, vw[2] = {vr[u][0], vr[u][1]};
+          float kf[8], vf[8];
+          Unpack<fp8_tag, 8>::run(kw, kf);
+          Unpack<fp8_tag, 8>::run(vw, vf);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            ((uint32_t*)&kn[u])[j] = (uint32_t)f32_to_elem_bits<XT>(kf[2 * j] * sk) | ((uint32_t)f32_to_elem_bits<XT>(kf[2 * j + 1] * sk) << 16);
+            ((uint32_t*)&vn[u])[j] = (uint32_t)f32_to_elem_bits<XT>(vf[2 * j] * sv) | ((uint32_t)f32_to_elem_bits<XT>(vf[2 * j + 1] * sv) << 16);
+          }
+        }
+        const int64_t dst = ((int64_t)b * stride + t) * row_elems + e;
+        *(uint4*)(kp + dst) = kn[u];
+        *(uint4*)(vp + dst) = vn[u];
+      }
+    }
+  }
+}
+
+const char* launch_dequant_pack_chunk(const void* k_pages, const void* v_pages, const void* k_new, const void* v_new,
+                                      const float* k_scale, const float* v_scale, const int32_t* cu_q, const int32_t* cache_seqlens,
+                                      const int32_t* block_table, int64_t bt_row_stride, void* kp, void* vp, int32_t* kv_starts,
+                                      int batch, int heads_kv, int dim, int page_size, int64_t n_pages, int stride, int x_dtype,
+                                      hipStream_t s) {
+  if (batch == 0) return nullptr;
+  const int64_t row_elems = (int64_t)heads_kv * dim;  // a multiple of 64: head dims are
+  const int64_t table_tokens64 = bt_row_stride * (int64_t)page_size;
+  const int table_tokens = table_tokens64 > INT_MAX ? INT_MAX : (int)table_tokens64;
+  int tpt_shift = 0;
+  while ((1 << tpt_shift) < row_elems / 8 && tpt_shift < 8) ++tpt_shift;
+  const dim3 grid((unsigned)((stride + 63) / 64), (unsigned)batch);
+#define MI355_LAUNCH_PACK(XT)                                                                                                  \
+  hipLaunchKernelGGL(dequant_pack_chunk_kernel<XT>, grid, dim3(256), 0, s, (const uint8_t*)k_pages, (const uint8_t*)v_pages,   \
+                     (const uint16_t*)k_new, (const uint16_t*)v_new, k_scale, v_scale, cu_q, cache_seqlens, block_table,       \
+                     bt_row_stride, (uint16_t*)kp, (uint16_t*)vp, kv_starts, row_elems, page_size, n_pages, stride, table_tokens, tpt_shift)
+  if (x_dtype == MI355_DT_BF16) MI355_LAUNCH_PACK(bf16_tag);
+  else MI355_LAUNCH_PACK(fp16_tag);
+#undef MI355_LAUNCH_PACK
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? nullptr : hipGetErrorString(e);
+}
+
 // Merge two attention results over disjoint key sets, given as fp32 rows with log2-domain log-sum-exp:
 //   out = (2^(lse_a - m) * o_a + 2^(lse_b - m) * o_b) / (2^(lse_a - m) + 2^(lse_b - m)),  m = max(lse_a, lse_b);
 // a row both sides left empty (-inf, -inf) becomes zero.  One thread per two head elements.
