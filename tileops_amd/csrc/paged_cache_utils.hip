@@ -407,8 +407,8 @@ __global__ __launch_bounds__(256) void dequant_pack_chunk_kernel(const uint8_t* 
   const float sk = k_scale[0], sv = v_scale[0];
   const int32_t* bt_row = block_table + (int64_t)b * bt_row_stride;
   // tpt threads per token row (the power of two that covers row_elems / 8, at most 256), 256 / tpt rows per round.
-  // Eight rounds at a time, every load of the eight issued before the first is used and none behind a branch (a row that is
-  // not of the kind a load is for reads a clamped neighbour and drops it): the kernel moves a few bytes per thread per
+  // Eight rounds at a time, every load of the eight issued before the first is used and none behind a per-row branch (in the one
+  // block of a sequence that holds both kinds of row, a row reads a clamped neighbour of the other kind and drops it): the kernel moves a few bytes per thread per
   // round, so what it needs is loads in flight, not arithmetic.
   const int sub = threadIdx.x >> tpt_shift, lane_e = threadIdx.x & ((1 << tpt_shift) - 1), rows_per_round = 256 >> tpt_shift;
   const int per_row = (int)(row_elems / 8);
@@ -418,26 +418,36 @@ __global__ __launch_bounds__(256) void dequant_pack_chunk_kernel(const uint8_t* 
   const bool one_page = (page_size & 63) == 0;
   const int blk0 = (int)blockIdx.x * 64;
   const int64_t phys_blk = physical_token(bt_row, min(blk0, last_old), page_size, n_pages) - min(blk0, last_old);
+  // A block of 64 tokens is all cached tokens, all chunk tokens, or (one block per sequence) both: the loads a block has
+  // no use for are not issued at all (the choice is the same for the whole workgroup).
+  const bool any_old = blk0 < n_old, any_new = t_end > n_old;
   for (int c = lane_e; c < per_row; c += 1 << tpt_shift) {  // (one trip unless a row is wider than 256 threads x 8 elements)
     const int64_t e = (int64_t)c * 8;
-    for (int t0 = (int)blockIdx.x * 64 + sub; t0 < t_end; t0 += UN * rows_per_round) {
-      int64_t phys[UN];
-#pragma unroll
-      for (int u = 0; u < UN; u++) {
-        const int tc = min(t0 + u * rows_per_round, last_old);
-        phys[u] = one_page ? phys_blk + tc : physical_token(bt_row, tc, page_size, n_pages);
-      }
+    for (int t0 = blk0 + sub; t0 < t_end; t0 += UN * rows_per_round) {
       u32x2 kr[UN], vr[UN];
       uint4 kn[UN], vn[UN];
+      if (any_old) {
+        int64_t phys[UN];
 #pragma unroll
-      for (int u = 0; u < UN; u++) {
-        const int t = t0 + u * rows_per_round;
-        const int64_t src_old = phys[u] * row_elems + e;
-        const int64_t src_new = ((int64_t)q0 + min(max(t - cached, 0), ql - 1)) * row_elems + e;  // chunk token t - cached
-        kr[u] = *(const u32x2*)(k_pages + src_old);
-        vr[u] = *(const u32x2*)(v_pages + src_old);
-        kn[u] = *(const uint4*)(k_new + src_new);
-        vn[u] = *(const uint4*)(v_new + src_new);
+        for (int u = 0; u < UN; u++) {
+          const int tc = min(t0 + u * rows_per_round, last_old);
+          phys[u] = one_page ? phys_blk + tc : physical_token(bt_row, tc, page_size, n_pages);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+          const int64_t src_old = phys[u] * row_elems + e;
+          kr[u] = *(const u32x2*)(k_pages + src_old);
+          vr[u] = *(const u32x2*)(v_pages + src_old);
+        }
+      }
+      if (any_new) {
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+          const int t = t0 + u * rows_per_round;
+          const int64_t src_new = ((int64_t)q0 + min(max(t - cached, 0), ql - 1)) * row_elems + e;  // chunk token t - cached
+          kn[u] = *(const uint4*)(k_new + src_new);
+          vn[u] = *(const uint4*)(v_new + src_new);
+        }
       }
 #pragma unroll
       for (int u = 0; u < UN; u++) {
