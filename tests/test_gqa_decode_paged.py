@@ -396,7 +396,7 @@ def test_many_query_rows_per_kv_head_share_their_stages(dtype, fp8, tol, q_len, 
         pytest.param(16, 32, 4, 128, False, id="bf16-ring-of-4"),
         pytest.param(32, 32, 4, 128, False, id="bf16-ring-of-8"),
         pytest.param(8, 64, 8, 64, False, id="bf16-head-dim-64-ring-of-2"),
-        pytest.param(32, 32, 4, 256, False, id="bf16-head-dim-256-ring-of-8-one-tile-per-barrier"),
+        pytest.param(32, 32, 4, 256, False, id="bf16-head-dim-256-ring-of-8"),
     ],
 )
 def test_ring_waves_walk_many_tiles_over_sequence_borders(num_split, q_len, heads, heads_kv, dim, fp8):

@@ -53,8 +53,8 @@ constexpr int kD = 128;       // default head dim (64 and 256 also run)
 // Single-row-block kernels with 128-byte rows (eight waves a CU) request the next tile only after the current one has
 // landed; asking earlier keeps more requests in flight per CU than the memory system rewards (measured: -4 %).
 constexpr bool kLateIssueNarrow = true;
-// Shared rings of four stages consume two tiles per barrier where two tiles of one sequence are left: one wait, one
-// barrier and one round of fetch requests per 64 tokens instead of per 32 (head dims up to 128; at 256 it measured 6 % slower).
+// Shared rings of four stages consume two tiles per barrier where two tiles of one sequence are left: one wait and one
+// barrier per 64 tokens instead of per 32.
 constexpr bool kPairSteps = true;
 
 // Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
@@ -1070,7 +1070,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   int u = 0, ring = 0, seg_count = 0;
   // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
   constexpr bool RESCALE_IN_LOOP = (SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2);
-  constexpr bool PAIRS = kPairSteps && SH && NS >= 4 && D <= 128 && RESCALE_IN_LOOP;
+  constexpr bool PAIRS = kPairSteps && SH && NS >= 4 && RESCALE_IN_LOOP;
+  // Head dim 256 has twice the fetch instructions per tile, and each holds its wave while the compute unit's address path
+  // takes it: a step's second fetch goes out between the step's tiles there instead of in one burst with the first
+  // (8 x 1024-token chunks on 32 K prefixes: 12.28 ms with the burst, 11.54 with one tile per barrier, 10.92 this way;
+  // at head dim 128 the burst is the faster by 1 %).
+  constexpr bool SPLIT_ISSUE = D == 256;
   constexpr int STEP = PAIRS ? NS / 2 : 1;  // tiles per barrier: half the ring is read while the other half is refilled
   while (u < n_units) {
     const int seg_first_j = cc.j;
@@ -1085,9 +1090,17 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
         // Past the barrier every wave's part of both tiles is in LDS, and every wave has finished reading the tiles before
         // u: their slots may be refilled.  Tile t goes to slot t % NS, so the request may run up to tile u + NS - 1.
         asm volatile("s_barrier" ::: "memory");
-        while (issued < n_units && issued - NS < u) {
-          issue(ci, issued & (NS - 1), ci_row);
-          if (++issued < n_units) advance();
+        const int u_step = u;
+        auto issue_one = [&]() __attribute__((always_inline)) {
+          if (issued < n_units && issued - NS < u_step) {
+            issue(ci, issued & (NS - 1), ci_row);
+            if (++issued < n_units) advance();
+          }
+        };
+        if constexpr (SPLIT_ISSUE) {
+          issue_one();
+        } else {
+          while (issued < n_units && issued - NS < u_step) issue_one();
         }
 #pragma nounroll
         for (int sub = 0; sub < step; ++sub) {  // (a loop, not two copies: the body is large)
@@ -1097,6 +1110,10 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
           ++cc.j;
           ring = (ring + 1) & (NS - 1);
           ++k;
+          if constexpr (SPLIT_ISSUE) issue_one();
+        }
+        if constexpr (SPLIT_ISSUE) {
+          while (issued < n_units && issued - NS < u_step) issue_one();  // (a step of one tile may have two slots to refill)
         }
       }
     }
