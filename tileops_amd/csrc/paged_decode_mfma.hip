@@ -1071,11 +1071,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
   constexpr bool RESCALE_IN_LOOP = (SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2);
   constexpr bool PAIRS = kPairSteps && SH && NS >= 4 && RESCALE_IN_LOOP;
-  // Head dim 256 has twice the fetch instructions per tile, and each holds its wave while the compute unit's address path
-  // takes it: a step's second fetch goes out between the step's tiles there instead of in one burst with the first
-  // (8 x 1024-token chunks on 32 K prefixes: 12.28 ms with the burst, 11.54 with one tile per barrier, 10.92 this way;
-  // at head dim 128 the burst is the faster by 1 %).
-  constexpr bool SPLIT_ISSUE = D == 256;
+  // A fetch instruction holds its wave while the compute unit's address path takes it.  Where a wave issues four or more
+  // of them per stage (head dim 256; fp8 and 64-byte-row rings of two) a step's second fetch goes out between the step's
+  // tiles instead of in one burst with the first: 8 x 1024-token chunks at head dim 256 on 32 K prefixes 12.28 ms with the
+  // burst, 11.54 with one tile per barrier, 10.92 this way; the eight-query-token fp8 configuration 152.9 -> 150.8 us.
+  // With two instructions per stage (16-bit rings of eight at head dim 128) the burst is the faster by 1 %.
+  constexpr bool SPLIT_ISSUE = IPSW >= 4;
   constexpr int STEP = PAIRS ? NS / 2 : 1;  // tiles per barrier: half the ring is read while the other half is refilled
   while (u < n_units) {
     const int seg_first_j = cc.j;
