@@ -650,6 +650,38 @@ def test_prefill_kernels_capture_into_a_graph_and_replay_on_new_values(rope):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("page, max_pages", [(64, 12), (16, 45)], ids=["page64", "page16-odd-page-count"])
+def test_fp8_cache_long_chunks_with_a_corrupt_cache_length_stay_inside_their_slot(page, max_pages):
+    """The dequantise-once route of long FP8-cache chunks under ``validate_inputs=False`` and a ``cache_seqlens`` entry of
+    ``2**31 - 5``: the packed slot of that sequence is filled from the pages its table row addresses and no further, its
+    chunk is appended nowhere, the output is finite, and the sane sequences match the oracle.  With 16-token pages and an odd
+    page count the slot is a few rows longer than the table row can address (slots are multiples of 32 rows)."""
+    require_gfx950()
+    H, Hkv, D, ql = 16, 4, 128, 260  # 1040 query rows per kv head
+    q_lens, old_lens = [ql, ql, 256], [300, 100, 0]
+    case = list(_case(q_lens, old_lens, H, Hkv, D, torch.float16, fp8=True, page=page, max_pages=max_pages, seed=19))
+    q, k_new, v_new, k_pages, v_pages, ks, vs, cu, cache, table = case
+    packed = native.prefill_paged_workspace(3, max(q_lens), sum(q_lens), H, Hkv, D, page, max_pages, torch.float16, FP8, native.KERNEL_AUTO)
+    assert packed >= 3 * max_pages * page * Hkv * D * 4  # the route under test
+    op = PrefillOp(batch=3, heads=H, heads_kv=Hkv, max_pages_per_req=max_pages, page_size=page, dim=D, is_causal=True, cache_dtype=FP8,
+                   validate_inputs=False)
+    dev = [t.to(DEV) for t in case]
+    bad = cache.clone()
+    bad[1] = 2**31 - 5
+    dev[8] = bad.to(DEV)
+    kp_before, vp_before = dev[3].clone(), dev[4].clone()
+    out = op(*dev, max(q_lens)).float().cpu()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    row1 = torch.cat([torch.arange(int(p) * page, (int(p) + 1) * page) for p in table[1]])
+    assert torch.equal(dev[3].cpu().view(torch.uint8)[row1], kp_before.cpu().view(torch.uint8)[row1])  # nothing appended
+    assert torch.equal(dev[4].cpu().view(torch.uint8)[row1], vp_before.cpu().view(torch.uint8)[row1])
+    ref_out, _, _ = ref_gqa_prefill_paged(*case, page_size=page, is_causal=True)
+    for lo, hi in ((0, ql), (2 * ql, 2 * ql + 256)):
+        torch.testing.assert_close(out[lo:hi], ref_out.float()[lo:hi], atol=8e-2, rtol=2e-2)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("kernel", [native.KERNEL_GENERIC, native.KERNEL_AUTO], ids=["general", "mfma"])
 @pytest.mark.parametrize("rope", [False, True])
 def test_a_cache_length_near_int_max_is_clamped_not_wrapped(kernel, rope):
