@@ -1075,8 +1075,9 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   // of them per stage (head dim 256; fp8 and 64-byte-row rings of two) a step's second fetch goes out between the step's
   // tiles instead of in one burst with the first: 8 x 1024-token chunks at head dim 256 on 32 K prefixes 12.28 ms with the
   // burst, 11.54 with one tile per barrier, 10.92 this way; the eight-query-token fp8 configuration 152.9 -> 150.8 us.
-  // With two instructions per stage (16-bit rings of eight at head dim 128) the burst is the faster by 1 %.
-  constexpr bool SPLIT_ISSUE = IPSW >= 4;
+  // With two instructions per stage and two tiles per step (16-bit rings of eight at head dim 128 on four stages) the burst
+  // was the faster by 1 %; on eight stages, four tiles per step, spreading wins again (413 -> 406 us).
+  constexpr bool SPLIT_ISSUE = IPSW >= 4 || NS == 8;
   constexpr int STEP = PAIRS ? NS / 2 : 1;  // tiles per barrier: half the ring is read while the other half is refilled
   while (u < n_units) {
     const int seg_first_j = cc.j;
@@ -1593,13 +1594,15 @@ const char* launch_t2(const DecodeParams& p, int* ws_prefix, bool skip_combine, 
   constexpr int NRB = D == 256 ? 1 : 2;  // == row_blocks_for(rows > 16, D)
   switch (ring_waves_for(p.rows, NRB, max_ring_for(D, Geom<KVT, D>::FP8))) {
     case 1: return launch_t4<QT, KVT, NRB, 2, NWU, 1, D>(p, ws_prefix, skip_combine, s);
-    case 2: return launch_t4<QT, KVT, NRB, SMALL ? 4 : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
+    // Stages per ring: as many as the LDS of a compute unit holds for its eight waves, up to eight -- half a ring is read
+    // per barrier while the other half is refilled, so eight stages mean one barrier per four tiles (8 x 512-token
+    // chunks on 4 K prefixes: 424 us with four stages, 406 with eight).
+    case 2: return launch_t4<QT, KVT, NRB, SMALL ? (Geom<KVT, D>::ROW == 64 ? 8 : 4) : 2, 2, 2, D>(p, ws_prefix, skip_combine, s);
     case 4:
-      if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
+      if constexpr (Geom<KVT, D>::NI >= 4) return launch_t4<QT, KVT, NRB, SMALL ? 8 : 4, 4, 4, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of four waves for this row width";
     default:
-      // (four stages: a ring of eight stages read four tiles per barrier measured 1.5 % faster at twice the LDS -- not taken)
-      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
+      if constexpr (!SMALL) return launch_t4<QT, KVT, NRB, Geom<KVT, D>::STAGE <= 16384 ? 8 : 4, 8, 8, D>(p, ws_prefix, skip_combine, s);
       return "MFMA kernel: no ring of eight waves for this row width";
   }
 }
