@@ -32,6 +32,7 @@ if str(ROOT) not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense bf16 matrix rate (the PV product and, for 16-bit caches, QK^T run in bf16)
 TRAFFIC_SOURCE = "profiles/hbm_traffic.json"
+DRY_RUN_MS = 25.0            # warm-up budget of the reference's timing protocol (benchmarks/timing.py)
 
 DESCRIPTIONS = {
     "c2": "Llama-3-8B-shape paged GQA decode, bf16 KV",
@@ -135,6 +136,23 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
     for i in range(max(warmup, 1)):  # the flush kernels are part of what has to be warm
         flush(i)
         out = op(*args)
+    torch.cuda.synchronize()
+    # The W calls asked for are followed by the dry-run phase of the reference's own timing protocol
+    # (benchmarks/timing.py:527-585): as many flushed calls as fit 25 ms, at least 10 and at most 200, counted from one
+    # calibration pass, the calls above included.  After idle the device runs its first tens of milliseconds slower (the
+    # FP8 configuration reads 100.5 us/call over twenty calls timed after five, 98.8 after the dry run), so without it a
+    # short run reports the ramp rather than the call.  Untimed, like the W calls; the timed region below is exactly K steps.
+    t0 = time.perf_counter()
+    for i in range(3):
+        flush(i)
+        op(*args)
+    torch.cuda.synchronize()
+    per_iter_ms = max((time.perf_counter() - t0) * 1e3 / 3, 1e-3)
+    warm_calls = max(warmup, 1) + 3
+    for i in range(max(min(max(int(DRY_RUN_MS / per_iter_ms), 10), 200) - warm_calls, 0)):
+        flush(i)
+        op(*args)
+        warm_calls += 1
     torch.cuda.synchronize()
     per_step_ms, wall = _timed_steps(lambda: op(*args), flush, steps)
     ms = sum(per_step_ms) / steps
@@ -243,6 +261,7 @@ def _run_config(name: str, steps: int, warmup: int, with_cpu: bool, kernel_key: 
             "kv_read_frac_of_peak_mean": gbs(kv_read, ms) / HBM_PEAK_GBS, "kv_read_frac_of_peak_median": gbs(kv_read, ms_median) / HBM_PEAK_GBS,
             "all_bytes_frac_of_peak_mean": gbs(total_bytes, ms) / HBM_PEAK_GBS,
             "event_pair_reads_when_empty_us": tare_ms * 1e3,
+            "untimed_calls_before_the_timed_steps": warm_calls,
         },
         # the attention kernel alone, cold: one launch per HIP-event pair, each after a cache flush (mean of the steps)
         "attention_kernel_us": kernel_ms * 1e3,
@@ -388,6 +407,8 @@ def main() -> None:
         "data": "synthetic", "config": {"workload": main_res["workload"], "kernel": main_res["kernel"],
                                         "process": "one per configuration" if len(names) > 1 and not a.in_process else "this one"},
         "roofline": main_res["roofline"],
+        "warmup_protocol": f"the {a.warmup} calls asked for, then the reference protocol's dry run (flushed calls for {DRY_RUN_MS:.0f} ms, 10 to 200): "
+                           f"{main_res['whole_call']['untimed_calls_before_the_timed_steps']} untimed calls in all before the {a.steps} timed steps",
     }
     for key in ("cpu_baseline", "cpu_baseline_sdpa_math", "parity", "mfma"):
         if key in main_res:
