@@ -416,10 +416,41 @@ def test_ring_waves_walk_many_tiles_over_sequence_borders(num_split, q_len, head
     assert torch.isfinite(out).all()
     tol = 3e-2 if fp8 else 2e-2
     torch.testing.assert_close(out.float().cpu(), ref.float(), atol=tol, rtol=tol)
-    # the same call cut into the default number of ranges (a tile or two per wave) differs by fp32 summation order only
+    # the same call cut into the default number of ranges (a tile or two per wave) differs by fp32 summation order and, in
+    # calls with this many query rows, by the partial rows' one rounding to the query's type
     auto = torch.ops.tileops_amd.gqa_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], q_len, heads, heads_kv, dim, 64,
                                                   dim ** -0.5, 0.0, True, 0, native.KERNEL_MFMA)
     torch.testing.assert_close(out.float(), auto.float(), atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("batch, many_rows", [(3, False), (9, True)])
+def test_partial_rows_are_fp32_for_few_query_rows_and_rounded_once_to_the_query_type_for_many(batch, many_rows):
+    """A range of the tile stream that ends inside a sequence leaves a partial row for the merge.  Calls with up to 4096
+    query rows keep those rows in fp32: cutting the stream differently moves the result by fp32 summation order, far below
+    one fp16 ulp.  Calls with more rows (multi-token decode of a batch, prefill chunks) store them in the query's type, as
+    the reference stores every partial (gqa_decode_paged.py:216-217,718-722): each partial is rounded once, the merged row
+    is a convex combination of them, so the result moves by at most one ulp of the largest value plus its own rounding."""
+    require_gfx950()
+    q_len, heads, heads_kv, dim = 8, 64, 8, 128
+    assert (heads_kv * q_len * (heads // heads_kv) * batch > 4096) == many_rows
+    lens = [2100, 8, 41, 700, 72, 9, 1500, 96, 4000][:batch]
+    case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, torch.float16, q_len=q_len, seed=131)
+    q, k, v, seqlens, table, _, _ = case
+    dev = [None if t is None else t.to(DEV) for t in case]
+    run = lambda ns: torch.ops.tileops_amd.gqa_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], q_len, heads, heads_kv, dim,
+                                                           64, dim ** -0.5, 0.0, True, ns, native.KERNEL_MFMA).float()
+    whole = run(1)   # one range per kv head: every sequence inside it, no partial rows at all
+    cut = run(0)     # the default: a few tiles per wave, most sequences cut many times
+    ref = ref_paged_gqa_decode(q, k, v, seqlens, table, page_size=64, is_causal=True)
+    torch.testing.assert_close(whole.cpu(), ref.float(), atol=5e-3, rtol=5e-3)
+    ulp = torch.finfo(torch.float16).eps  # of values in [1, 2)
+    vmax = float(torch.nan_to_num(v.float(), nan=0.0).abs().max())  # (unaddressed tokens hold NaN)
+    outmax = float(whole.abs().max())
+    diff = (cut - whole).abs().max().item()
+    if many_rows:
+        assert diff <= ulp * (0.5 * vmax + outmax), diff
+    else:
+        assert diff <= ulp * outmax, diff  # fp32 values a hair apart (summation order, the probabilities' own rounding), rounded to fp16
 
 
 @pytest.mark.parametrize("softcap", [0.0, 30.0])

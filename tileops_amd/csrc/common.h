@@ -48,7 +48,7 @@ struct DecodeParams {
   const float* init_o;
   const float* init_lse;
   void* out;
-  float* part_o;    // workspace: normalised partial outputs, fp32
+  float* part_o;    // workspace: normalised partial outputs, fp32 (or rows of the query's 16-bit type: part16)
   float* part_lse;  // workspace: log2-domain log-sum-exp per partial (-inf = empty)
   int batch, q_len, heads, heads_kv, dim, page_size;
   int group;        // heads / heads_kv
@@ -66,6 +66,7 @@ struct DecodeParams {
   int split_tokens;
   // MFMA kernel: even partition of the KV tile stream
   int n_parts;
+  int part16;        // partial output rows are stored in the query's 16-bit type (the dtype of the reference's partials)
 };
 
 // Context length of sequence b: per-sequence array (paged cache) or one value for all (contiguous cache), clamped to

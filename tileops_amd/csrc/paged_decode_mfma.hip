@@ -12,7 +12,8 @@
 //    real_seqlen_kv, so all
 //    compute units get the same number of tiles whatever the length distribution, and nothing is read back
 //    to the host.  A range that covers a whole sequence writes the output directly; a range that starts or
-//    ends inside a sequence writes an fp32 partial (at most two per wave) that the combine kernel merges.
+//    ends inside a sequence writes a partial row and its fp32 log-sum-exp (at most two per wave) that the combine kernel
+//    merges; the rows are fp32, or the query's 16-bit type in calls with more than 4096 query rows (launch_mfma).
 //  * Page gather = 128-bit direct-to-LDS loads (global_load_lds_dwordx4) with the non-temporal hint, 1 KiB
 //    per wave instruction covering whole 128-, 256- or 512-byte K/V rows (head dim x element size), NS stages per wave in
 //    flight, waited on with s_waitcnt vmcnt.  The LDS image is XOR-swizzled by choosing which 16-byte chunk
@@ -100,6 +101,14 @@ template <> struct Mma<fp16_tag> {
     return __builtin_bit_cast(uint32_t, r);
   }
 };
+
+template <typename QT> __device__ __forceinline__ f32x2 unpack2(uint32_t w);
+template <> __device__ __forceinline__ f32x2 unpack2<bf16_tag>(uint32_t w) {
+  return f32x2{__builtin_bit_cast(float, w << 16), __builtin_bit_cast(float, w & 0xffff0000u)};
+}
+template <> __device__ __forceinline__ f32x2 unpack2<fp16_tag>(uint32_t w) {
+  return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+}
 
 // 16x16 tile of 128-deep dot products of e4m3fn bytes (v_mfma_f32_16x16x128_f8f6f4, no block scales): lane (c, g)
 // supplies 32 bytes of row c of each operand.  Which 32 of the 128 depth positions those are is the same function of g
@@ -1018,9 +1027,21 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
         }
       } else {
         int64_t grow = ((int64_t)(2 * part + which) * p.heads_kv + kvh) * p.rows + r;
-        float* pp = p.part_o + grow * D;
+        if (p.part16) {
+          uint16_t* pp = (uint16_t*)p.part_o + grow * D;
 #pragma unroll
-        for (int db = 0; db < NDB; db++) *(f32x4*)(pp + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+          for (int db = 0; db < NDB; db++) {
+            f32x4 o = o_acc[rb][db] * inv;
+            u32x2 w;
+            w[0] = Mma<QT>::pack(o[0], o[1]);
+            w[1] = Mma<QT>::pack(o[2], o[3]);
+            *(u32x2*)(pp + 16 * db + 4 * g) = w;
+          }
+        } else {
+          float* pp = p.part_o + grow * D;
+#pragma unroll
+          for (int db = 0; db < NDB; db++) *(f32x4*)(pp + 16 * db + 4 * g) = o_acc[rb][db] * inv;
+        }
         if (g == 0) p.part_lse[grow] = l_tot > 0.f ? m_run[rb] + log2f(l_tot) : -INFINITY;
       }
     }
@@ -1160,7 +1181,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 
 // Merge the partials of sequences that span more than one partition, and zero-fill empty sequences.
 //   lse = log2 sum_s 2^(lse_s - max) + max ; O = sum_s 2^(lse_s - lse) * O_s   (reference combine,
-//   src/tileops/kernels/attention/gqa_decode_paged.py:344-374), on fp32 partials.
+//   src/tileops/kernels/attention/gqa_decode_paged.py:344-374), on fp32 or 16-bit partial rows (DecodeParams::part16) and fp32 log-sum-exps.
 // Four waves work on one (sequence, kv head, query row) at a time.  Every wave forms the maximum and the sum of
 // weights over all partitions of the sequence (lane i fetches the LSE of partition i, two wave reductions per 64);
 // the weighted sum of the partial rows is split over the waves (wave w takes partitions w, w+4, ...), eight
@@ -1169,6 +1190,18 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 // sequence spread over hundreds of partitions (batch-1 long-context decode) is then merged in a few load round
 // trips instead of one per partition.  64*kCombineWaves threads; the launcher takes the one-wave instance when the
 // average sequence spans at most eight partitions.
+// One lane's two elements of a partial output row: fp32, or the query's 16-bit type widened.
+template <typename QT>
+__device__ __forceinline__ f32x2 load_part2(const DecodeParams& p, int64_t slot, int hd, int dl) {
+  if (p.part16) return unpack2<QT>(*(const uint32_t*)((const uint16_t*)p.part_o + slot * hd + dl));
+  return *(const f32x2*)(p.part_o + slot * hd + dl);
+}
+// The same load with the 16-bit pair left as bits in element 0 (many loads in flight, widened when consumed).
+__device__ __forceinline__ f32x2 load_part2_raw(const DecodeParams& p, int64_t slot, int hd, int dl) {
+  if (p.part16) return f32x2{__builtin_bit_cast(float, *(const uint32_t*)((const uint16_t*)p.part_o + slot * hd + dl)), 0.f};
+  return *(const f32x2*)(p.part_o + slot * hd + dl);
+}
+
 template <typename QT, int kCombineWaves>
 __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __restrict__ ws_prefix, f32x2 (*red)[64], int b, int row_all, int4 rec,
                                             int wave);
@@ -1249,7 +1282,7 @@ __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __
   // this wave's first eight partial rows go out together with the LSEs, before any weight is known
   f32x2 rows[PRE];
 #pragma unroll
-  for (int i = 0; i < PRE; i++) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + wave + nw * i, p_last)) * hd + dl);
+  for (int i = 0; i < PRE; i++) rows[i] = load_part2<QT>(p, slot_of(min(p_first + wave + nw * i, p_last)), hd, dl);
   // lane i keeps the LSE of partition i of the first 64 (all of them, as a rule); further ones are re-read
   const float lse0 = (p_first + lane <= p_last && owns_tiles(p_first + lane)) ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
   float M = lse0;
@@ -1284,7 +1317,7 @@ __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __
         const int idx = wave + nw * (i0 + i), pp = p_first + idx;  // wave-uniform
         if (idx < 64) wt[i] = __shfl(w0, idx, 64);
         else wt[i] = (pp <= p_last && owns_tiles(pp)) ? fast_exp2(p.part_lse[slot_of(pp)] - M) : 0.f;
-        if (i0 > 0) rows[i] = *(const f32x2*)(p.part_o + slot_of(min(pp, p_last)) * hd + dl);
+        if (i0 > 0) rows[i] = load_part2<QT>(p, slot_of(min(pp, p_last)), hd, dl);
       }
 #pragma unroll
       for (int i = 0; i < PRE; i++)
@@ -1332,7 +1365,7 @@ __device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int 
     live[r] = row0 + r < row_end && row_all - kvh * p.rows < q_rows;  // (packed queries: this sequence may have fewer rows)
     auto slot_of = [&](int pp) { return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all; };
 #pragma unroll
-    for (int i = 0; i < PRE; i++) rows[r][i] = *(const f32x2*)(p.part_o + slot_of(min(p_first + i, p_last)) * hd + dl);
+    for (int i = 0; i < PRE; i++) rows[r][i] = load_part2_raw(p, slot_of(min(p_first + i, p_last)), hd, dl);
     lse[r] = lane < n ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
   }
 #pragma unroll
@@ -1355,9 +1388,10 @@ __device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int 
 #pragma unroll
     for (int i = 0; i < PRE; i++) {
       const float wt = __shfl(w0, i, 64);
+      const f32x2 row = p.part16 ? unpack2<QT>(__builtin_bit_cast(uint32_t, rows[r][i][0])) : rows[r][i];
       if (wt != 0.f) {  // an unwritten slot may hold anything, NaN included
-        acc0 = fmaf(wt, rows[r][i][0], acc0);
-        acc1 = fmaf(wt, rows[r][i][1], acc1);
+        acc0 = fmaf(wt, row[0], acc0);
+        acc1 = fmaf(wt, row[1], acc1);
       }
     }
     const float inv = W > 0.f ? 1.0f / W : 0.f;
@@ -1648,6 +1682,15 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   p.negate_q = signed_scale < 0.f ? 1 : 0;
   signed_scale = fabsf(signed_scale);
   if (!(p.softcap > 0.f) && signed_scale < 1e-30f) signed_scale = 1e-30f;
+  // Calls with many query rows (multi-token decode, prefill chunks) keep their partial rows in the query's 16-bit type, as the
+  // reference does for every call (its Output_partial has the op's dtype, gqa_decode_paged.py:216-217,718-722): half the
+  // bytes written by the attention kernel and read by the merge.  The log-sum-exps stay fp32, and so do the rows of
+  // single-token decode.  (The sixteen-wave merge of very long single sequences reads fp32 rows only.)
+  {
+    const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
+    const bool wide = (int64_t)p.n_parts > 64 * (int64_t)p.batch;
+    p.part16 = (!wide && rows_all * p.batch > 4096) ? 1 : 0;
+  }
   size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
   char* ws = (char*)p_in.part_o;
   p.part_o = (float*)ws;
