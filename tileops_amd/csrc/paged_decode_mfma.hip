@@ -1341,12 +1341,10 @@ __device__ __forceinline__ void combine_row(const DecodeParams& p, const int* __
   store(acc0 * inv, acc1 * inv, W > 0.f ? M + log2f(W) : -INFINITY);
 }
 
-// R rows of one sequence merged by one wave, every load of every row issued before the first is consumed: with tens of
-// thousands of rows (eight query tokens x group 8 x 32 sequences) the merge kernel is otherwise two rounds of workgroups,
-// each a chain of three dependent reads.  At most eight partials per row, every partition owning tiles (the caller checks).
-template <typename QT, int R>
-__device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int b, int row0, int row_end, int4 rec) {
+template <typename QT, int R, bool P16>
+__device__ __forceinline__ void combine_rows_at_once_t(const DecodeParams& p, int b, int row0, int row_end, int4 rec) {
   constexpr int PRE = 8;
+  constexpr int ES = P16 ? 2 : 4;  // bytes per element of a partial row
   const int lane = threadIdx.x & 63;
   const int hd = p.dim;
   const bool owns = 2 * lane < hd;
@@ -1355,40 +1353,70 @@ __device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int 
   const bool first_in_slot1 = (rec.w & 1) != 0;
   const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
   const int q_rows = p.cu_q ? q_len_of(p, b) * p.group : p.rows;
-  f32x2 rows[R][PRE];
-  float lse[R];
-  bool live[R];
+  // Addresses: partition i's copy of row row0 is formed once (wave-uniform, 64-bit); the wave's other rows lie whole rows
+  // behind it, and a lane adds its two elements' offset.  (Formed per load, the 64-bit products were 2000 scalar
+  // instructions a wave -- the kernel was bound by them.)
+  const uint32_t row_bytes = (uint32_t)hd * ES, lane_off = (uint32_t)dl * ES;
+  const char* base[PRE];
 #pragma unroll
-  for (int r = 0; r < R; r++) {
-    const int row_all = min(row0 + r, row_end - 1);
-    const int kvh = row_all / p.rows;
-    live[r] = row0 + r < row_end && row_all - kvh * p.rows < q_rows;  // (packed queries: this sequence may have fewer rows)
-    auto slot_of = [&](int pp) { return (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row_all; };
-#pragma unroll
-    for (int i = 0; i < PRE; i++) rows[r][i] = load_part2_raw(p, slot_of(min(p_first + i, p_last)), hd, dl);
-    lse[r] = lane < n ? p.part_lse[slot_of(p_first + lane)] : -INFINITY;
+  for (int i = 0; i < PRE; i++) {
+    const int pp = min(p_first + i, p_last);
+    const int64_t slot = (int64_t)(2 * pp + ((pp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row0;
+    base[i] = uni_ptr((const char*)p.part_o + slot * (int64_t)row_bytes);
   }
+  const int lp = min(p_first + lane, p_last);
+  const float* lse_lane = p.part_lse + ((int64_t)(2 * lp + ((lp == p_first && first_in_slot1) ? 1 : 0)) * rows_all + row0);
+  const int last_r = row_end - 1 - row0;  // rows past the workgroup's range re-read its last row and are not stored
+  uint32_t raw[R][PRE][P16 ? 1 : 2];
+  float lse[R];
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    if (!live[r]) continue;
-    const int row_all = row0 + r;
-    const int kvh = row_all / p.rows, rr = row_all - kvh * p.rows;
-    const int s = rr / p.group, gi = rr - s * p.group;
-    const int64_t orow = (q_row0_of(p, b) + s) * p.heads + kvh * p.group + gi;
-    float M = lse[r];
-#pragma unroll
-    for (int m = 1; m < PRE; m <<= 1) M = fmaxf(M, __shfl_xor(M, m, 64));  // the first eight lanes hold the LSEs
-    M = __shfl(M, 0, 64);
-    const float w0 = (M != -INFINITY && lse[r] != -INFINITY) ? fast_exp2(lse[r] - M) : 0.f;
-    float W = w0;
-#pragma unroll
-    for (int m = 1; m < PRE; m <<= 1) W += __shfl_xor(W, m, 64);
-    W = __shfl(W, 0, 64);
-    float acc0 = 0.f, acc1 = 0.f;
+    const uint32_t roff = (uint32_t)min(r, last_r) * row_bytes + lane_off;
 #pragma unroll
     for (int i = 0; i < PRE; i++) {
-      const float wt = __shfl(w0, i, 64);
-      const f32x2 row = p.part16 ? unpack2<QT>(__builtin_bit_cast(uint32_t, rows[r][i][0])) : rows[r][i];
+      if constexpr (P16) {
+        raw[r][i][0] = *(const uint32_t*)(base[i] + roff);
+      } else {
+        const u32x2 w = *(const u32x2*)(base[i] + roff);
+        raw[r][i][0] = w[0];
+        raw[r][i][1] = w[1];
+      }
+    }
+    lse[r] = lane < n ? lse_lane[min(r, last_r)] : -INFINITY;
+  }
+  // row indices of row0, stepped from row to row (divisions cost more than everything else a row needs)
+  int kvh = row0 / p.rows, rr = row0 - kvh * p.rows, s = rr / p.group, gi = rr - s * p.group;
+  const int64_t q_row0 = q_row0_of(p, b);
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const bool live = r <= last_r && rr < q_rows;  // (packed queries: this sequence may have fewer rows)
+    const int64_t orow = (q_row0 + s) * p.heads + kvh * p.group + gi;
+    if (++gi == p.group) {
+      gi = 0;
+      ++s;
+    }
+    if (++rr == p.rows) {
+      rr = 0;
+      s = 0;
+      gi = 0;
+      ++kvh;
+    }
+    if (!live) continue;
+    // the first eight lanes hold the log-sum-exps: as wave-uniform values, so that nothing below crosses lanes
+    float l[PRE], M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+      l[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lse[r]), i));
+      M = fmaxf(M, l[i]);
+    }
+    float W = 0.f, acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+      const float wt = (M != -INFINITY && l[i] != -INFINITY) ? fast_exp2(l[i] - M) : 0.f;
+      W += wt;
+      f32x2 row;
+      if constexpr (P16) row = unpack2<QT>(raw[r][i][0]);
+      else row = f32x2{__builtin_bit_cast(float, raw[r][i][0]), __builtin_bit_cast(float, raw[r][i][1])};
       if (wt != 0.f) {  // an unwritten slot may hold anything, NaN included
         acc0 = fmaf(wt, row[0], acc0);
         acc1 = fmaf(wt, row[1], acc1);
@@ -1403,6 +1431,15 @@ __device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int 
       *((uint32_t*)((uint16_t*)p.out + orow * hd) + (dl >> 1)) = Mma<QT>::pack(acc0 * inv, acc1 * inv);
     }
   }
+}
+
+// R rows of one sequence merged by one wave, every load of every row issued before the first is consumed: with tens of
+// thousands of rows (eight query tokens x group 8 x 32 sequences) the merge kernel is otherwise two rounds of workgroups,
+// each a chain of three dependent reads.  At most eight partials per row, every partition owning tiles (the caller checks).
+template <typename QT, int R>
+__device__ __forceinline__ void combine_rows_at_once(const DecodeParams& p, int b, int row0, int row_end, int4 rec) {
+  if (p.part16) combine_rows_at_once_t<QT, R, true>(p, b, row0, row_end, rec);
+  else combine_rows_at_once_t<QT, R, false>(p, b, row0, row_end, rec);
 }
 
 // The same merge for calls whose sequences span very many partitions each (batch-1 long-context decode).
