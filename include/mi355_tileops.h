@@ -93,8 +93,8 @@ int mi355_gqa_paged_decode_workspace(int batch, int q_len, int heads, int heads_
  *   out          [batch, q_len, heads, dim] q_dtype
  *   workspace    >= the size mi355_gqa_paged_decode_workspace() reports for the same arguments, 256-byte aligned.
  *                It holds what the reference keeps in glse / Output_partial (gqa_decode_paged.py:718-722): log-sum-exps in
- *                fp32; partial output rows in fp32, or -- on the MFMA kernel, in calls of more than 4096 query rows
- *                (batch * q_len * heads) -- in q_dtype, the type the reference gives every partial (:216-217)
+ *                fp32; partial output rows in fp32, or -- on the MFMA kernel, with q_len > 1 and more than 4096 query
+ *                rows (batch * q_len * heads) -- in q_dtype, the type the reference gives every partial (:216-217)
  *   sm_scale     softmax scale applied to q.k  (the op passes dim**-0.5 unless overridden, gqa.py:81-82)
  *   softcap      0 = off, else scores := softcap * tanh(scores / softcap)  (online_softmax.py:153-173)
  *   causal       with q_len > 1: query i sees key j iff j <= i + (seqlens[b] - q_len)  (gqa.py:558-562)

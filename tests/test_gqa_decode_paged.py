@@ -423,17 +423,18 @@ def test_ring_waves_walk_many_tiles_over_sequence_borders(num_split, q_len, head
     torch.testing.assert_close(out.float(), auto.float(), atol=tol, rtol=tol)
 
 
-@pytest.mark.parametrize("batch, many_rows", [(3, False), (9, True)])
-def test_partial_rows_are_fp32_for_few_query_rows_and_rounded_once_to_the_query_type_for_many(batch, many_rows):
-    """A range of the tile stream that ends inside a sequence leaves a partial row for the merge.  Calls with up to 4096
-    query rows keep those rows in fp32: cutting the stream differently moves the result by fp32 summation order, far below
-    one fp16 ulp.  Calls with more rows (multi-token decode of a batch, prefill chunks) store them in the query's type, as
-    the reference stores every partial (gqa_decode_paged.py:216-217,718-722): each partial is rounded once, the merged row
+@pytest.mark.parametrize("batch, q_len, many_rows", [(3, 8, False), (9, 8, True), (70, 1, False)])
+def test_partial_rows_are_fp32_for_few_query_rows_and_rounded_once_to_the_query_type_for_many(batch, q_len, many_rows):
+    """A range of the tile stream that ends inside a sequence leaves a partial row for the merge.  Single-token decode, and
+    multi-token calls with up to 4096 query rows, keep those rows in fp32: cutting the stream differently moves the result by
+    fp32 summation order, far below one fp16 ulp.  Multi-token calls with more rows (verify steps of a batch, prefill chunks)
+    store them in the query's type, as the reference stores every partial (gqa_decode_paged.py:216-217,718-722): each partial is rounded once, the merged row
     is a convex combination of them, so the result moves by at most one ulp of the largest value plus its own rounding."""
     require_gfx950()
-    q_len, heads, heads_kv, dim = 8, 64, 8, 128
-    assert (heads_kv * q_len * (heads // heads_kv) * batch > 4096) == many_rows
-    lens = [2100, 8, 41, 700, 72, 9, 1500, 96, 4000][:batch]
+    heads, heads_kv, dim = 64, 8, 128
+    assert (q_len > 1 and heads * q_len * batch > 4096) == many_rows
+    assert heads * q_len * batch > 4096 or batch == 3  # (the single-token case is past the row count, and still fp32)
+    lens = ([2100, 8, 41, 700, 72, 9, 1500, 96, 4000] + [(97 * i) % 900 + 33 for i in range(61)])[:batch]
     case = _ragged_case(len(lens), heads, heads_kv, dim, 64, lens, torch.float16, q_len=q_len, seed=131)
     q, k, v, seqlens, table, _, _ = case
     dev = [None if t is None else t.to(DEV) for t in case]
@@ -443,6 +444,7 @@ def test_partial_rows_are_fp32_for_few_query_rows_and_rounded_once_to_the_query_
     cut = run(0)     # the default: a few tiles per wave, most sequences cut many times
     ref = ref_paged_gqa_decode(q, k, v, seqlens, table, page_size=64, is_causal=True)
     torch.testing.assert_close(whole.cpu(), ref.float(), atol=5e-3, rtol=5e-3)
+    assert whole.shape == cut.shape == ref.shape
     ulp = torch.finfo(torch.float16).eps  # of values in [1, 2)
     vmax = float(torch.nan_to_num(v.float(), nan=0.0).abs().max())  # (unaddressed tokens hold NaN)
     outmax = float(whole.abs().max())

@@ -13,7 +13,7 @@
 //    compute units get the same number of tiles whatever the length distribution, and nothing is read back
 //    to the host.  A range that covers a whole sequence writes the output directly; a range that starts or
 //    ends inside a sequence writes a partial row and its fp32 log-sum-exp (at most two per wave) that the combine kernel
-//    merges; the rows are fp32, or the query's 16-bit type in calls with more than 4096 query rows (launch_mfma).
+//    merges; the rows are fp32, or the query's 16-bit type in multi-token calls with more than 4096 query rows (launch_mfma).
 //  * Page gather = 128-bit direct-to-LDS loads (global_load_lds_dwordx4) with the non-temporal hint, 1 KiB
 //    per wave instruction covering whole 128-, 256- or 512-byte K/V rows (head dim x element size), NS stages per wave in
 //    flight, waited on with s_waitcnt vmcnt.  The LDS image is XOR-swizzled by choosing which 16-byte chunk
@@ -1726,7 +1726,7 @@ const char* launch_mfma(const DecodeParams& p_in, int q_dtype, int kv_dtype, boo
   {
     const int64_t rows_all = (int64_t)p.heads_kv * p.rows;
     const bool wide = (int64_t)p.n_parts > 64 * (int64_t)p.batch;
-    p.part16 = (!wide && rows_all * p.batch > 4096) ? 1 : 0;
+    p.part16 = (!wide && p.rows > p.group && rows_all * p.batch > 4096) ? 1 : 0;  // (rows == group: one query token)
   }
   size_t slots = (size_t)2 * p.n_parts * p.heads_kv * p.rows;
   char* ws = (char*)p_in.part_o;
