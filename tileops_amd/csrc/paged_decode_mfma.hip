@@ -57,6 +57,7 @@ constexpr bool kLateIssueNarrow = true;
 // Shared rings of four stages consume two tiles per barrier where two tiles of one sequence are left: one wait and one
 // barrier per 64 tokens instead of per 32.
 constexpr bool kPairSteps = true;
+constexpr bool kKPrefetch = true;
 
 // Row groups (16*NRB query rows each) per kv head, and the same rounded up to whole rings of SHW waves: a ring may
 // hold row groups past the last query row, which load nothing, mask everything and store nothing.
@@ -729,6 +730,12 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   // The same ring with an FP8 cache: the 32 registers of V^T bytes are read inside the value step as well, four 16-column
   // blocks at a time, and widened there.
   constexpr bool LATE_VREAD8 = FP8 && D == 256 && SHW == 8;
+  // 16-bit rings of two row blocks at head dims up to 128, several tiles per barrier: the K operands of a step's next tile
+  // are read from LDS behind this tile's score products (the registers of the operands they replace are free by then), so
+  // that they land under the softmax instead of in front of the next tile's first product.
+  constexpr bool KPRE = kKPrefetch && !FP8 && NRB == 2 && SH && NS >= 4 && D <= 128 && !LATE_VREAD;
+  u32x4 k_held[2][KPRE ? NJ : 1];  // the K operands of the tile at hand, carried from tile to tile
+  bool have_k_pre = false;
   u32x4 va_op[(LATE_V || LATE_VREAD) ? 1 : NDB];
   i32x2 vraw[(LATE_V && !LATE_VREAD8) ? NDB : 1];
   u32x4 pk[NRB];
@@ -742,7 +749,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     if constexpr (NRB != 1 || LATE_VREAD) asm volatile("" : "+v"(a));
     return a;
   };
-  auto score_step = [&](const uint32_t SOFF, const Cursor& cu) __attribute__((always_inline)) -> bool {
+  auto score_step = [&](const uint32_t SOFF, const Cursor& cu, const uint32_t NEXT_SOFF = 0xffffffffu) __attribute__((always_inline)) -> bool {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
     u32x4 ka_op[2][NJ];
@@ -752,7 +759,14 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 #pragma unroll
     for (int i = 0; i < NKA; i++) kb[i] = in_slot(kaddr[i], SOFF);
     if constexpr (!FP8) {
-      if constexpr (!LATE_VREAD) {
+      if constexpr (KPRE) {
+        if (!have_k_pre) {
+#pragma unroll
+          for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) k_held[tb][j] = *LDS_AT(u32x4, kb[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
+        }
+      } else if constexpr (!LATE_VREAD) {
 #pragma unroll
         for (int tb = 0; tb < 2; tb++)
 #pragma unroll
@@ -857,8 +871,23 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
         for (int rb = 0; rb < NRB; rb++)
 #pragma unroll
           for (int tb = 0; tb < 2; tb++) {
-            s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
+            if constexpr (KPRE) s_acc[tb][rb] = Mma<QT>::run(k_held[tb][j], qreg[rb][j], s_acc[tb][rb]);
+            else s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
           }
+      if constexpr (KPRE) {
+        have_k_pre = NEXT_SOFF != 0xffffffffu;
+        if (have_k_pre) {
+          __builtin_amdgcn_sched_barrier(0);  // behind the products above
+          uint32_t kn[NKA];
+#pragma unroll
+          for (int i = 0; i < NKA; i++) kn[i] = in_slot(kaddr[i], NEXT_SOFF);
+#pragma unroll
+          for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) k_held[tb][j] = *LDS_AT(u32x4, kn[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
     if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
     // ---- online softmax (exp2 domain), lane-local per query row -------------------------------------------
@@ -1088,6 +1117,9 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
       return score_step((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
     }
   };
+  auto run_score_step_pre = [&](int ring, bool more) __attribute__((always_inline)) -> bool {
+    return score_step((uint32_t)ring * G::STAGE, cc, more ? (uint32_t)((ring + 1) & (NS - 1)) * G::STAGE : 0xffffffffu);
+  };
   int u = 0, ring = 0, seg_count = 0;
   // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
   constexpr bool RESCALE_IN_LOOP = (SH && (D <= 128 || SHW == 8)) || (FP8 && NRB == 2);
@@ -1127,7 +1159,10 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
         }
 #pragma nounroll
         for (int sub = 0; sub < step; ++sub) {  // (a loop, not two copies: the body is large)
-          if (__builtin_expect(run_score_step(ring), 0)) rescale();
+          bool moved_;
+          if constexpr (KPRE) moved_ = run_score_step_pre(ring, sub + 1 < step);
+          else moved_ = run_score_step(ring);
+          if (__builtin_expect(moved_, 0)) rescale();
           value_step((uint32_t)ring * G::STAGE);
           ++u;
           ++cc.j;
