@@ -734,7 +734,9 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
   // are read from LDS behind this tile's score products (the registers of the operands they replace are free by then), so
   // that they land under the softmax instead of in front of the next tile's first product.
   constexpr bool KPRE = kKPrefetch && !FP8 && NRB == 2 && SH && NS >= 4 && D <= 128 && !LATE_VREAD;
-  u32x4 k_held[2][KPRE ? NJ : 1];  // the K operands of the tile at hand, carried from tile to tile
+  // Head dim 256 on rings of eight (K read in two halves of the head dim): the first half is carried the same way.
+  constexpr bool KPRE2 = kKPrefetch && LATE_VREAD && NRB == 1 && NS >= 4;
+  u32x4 k_held[2][KPRE ? NJ : (KPRE2 ? NJ / 2 : 1)];  // the K operands of the tile at hand, carried from tile to tile
   bool have_k_pre = false;
   u32x4 va_op[(LATE_V || LATE_VREAD) ? 1 : NDB];
   i32x2 vraw[(LATE_V && !LATE_VREAD8) ? NDB : 1];
@@ -749,7 +751,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
     if constexpr (NRB != 1 || LATE_VREAD) asm volatile("" : "+v"(a));
     return a;
   };
-  auto score_step = [&](const uint32_t SOFF, const Cursor& cu, const uint32_t NEXT_SOFF = 0xffffffffu) __attribute__((always_inline)) -> bool {
+  auto score_step = [&](const uint32_t SOFF, const Cursor& cu, const uint32_t NEXT_SOFF = 0u, const bool more = false) __attribute__((always_inline)) -> bool {
     const int tok0 = cu.j * kCT;
     // ---- all LDS reads of the stage go out first: 8 K operands, 8 V^T operands (+ scales) ----------------
     u32x4 ka_op[2][NJ];
@@ -845,24 +847,52 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
                                            qreg[rb][part * NCH + 2 * h + 1], s_acc[tb][rb]);
     } else if constexpr (LATE_VREAD) {
       // the K operands in two halves of the head dim (32 registers each): read, multiply, read, multiply
-#pragma unroll
-      for (int hf = 0; hf < 2; hf++) {
-        u32x4 kh[2][NJ / 2];
+      auto read_half = [&](int hf, const uint32_t* base, u32x4 (*dst)[KPRE2 ? NJ / 2 : NJ / 2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int tb = 0; tb < 2; tb++)
 #pragma unroll
           for (int jj = 0; jj < NJ / 2; jj++) {
             const int j = hf * (NJ / 2) + jj;
-            kh[tb][jj] = *LDS_AT(u32x4, kb[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
+            dst[tb][jj] = *LDS_AT(u32x4, base[j % NKA] + (tb * HALF + (j / NKA) * (NKA * 64)));
           }
+      };
+      if constexpr (KPRE2) {
+        u32x4 kh1[2][NJ / 2];
+        if (!have_k_pre) read_half(0, kb, k_held);
+        read_half(1, kb, kh1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jj = 0; jj < NJ / 2; jj++)
 #pragma unroll
-          for (int rb = 0; rb < NRB; rb++)
-#pragma unroll
-            for (int tb = 0; tb < 2; tb++) s_acc[tb][rb] = Mma<QT>::run(kh[tb][jj], qreg[rb][hf * (NJ / 2) + jj], s_acc[tb][rb]);
+          for (int tb = 0; tb < 2; tb++) s_acc[tb][0] = Mma<QT>::run(k_held[tb][jj], qreg[0][jj], s_acc[tb][0]);
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jj = 0; jj < NJ / 2; jj++)
+#pragma unroll
+          for (int tb = 0; tb < 2; tb++) s_acc[tb][0] = Mma<QT>::run(kh1[tb][jj], qreg[0][NJ / 2 + jj], s_acc[tb][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        have_k_pre = more;
+        if (have_k_pre) {
+          uint32_t kn[NKA];
+#pragma unroll
+          for (int i = 0; i < NKA; i++) kn[i] = in_slot(kaddr[i], NEXT_SOFF);
+          read_half(0, kn, k_held);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+          u32x4 kh[2][NJ / 2];
+          read_half(hf, kb, kh);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int jj = 0; jj < NJ / 2; jj++)
+#pragma unroll
+            for (int rb = 0; rb < NRB; rb++)
+#pragma unroll
+              for (int tb = 0; tb < 2; tb++) s_acc[tb][rb] = Mma<QT>::run(kh[tb][jj], qreg[rb][hf * (NJ / 2) + jj], s_acc[tb][rb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     } else {
 #pragma unroll
@@ -875,7 +905,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
             else s_acc[tb][rb] = Mma<QT>::run(ka_op[tb][j], qreg[rb][j], s_acc[tb][rb]);
           }
       if constexpr (KPRE) {
-        have_k_pre = NEXT_SOFF != 0xffffffffu;
+        have_k_pre = more;
         if (have_k_pre) {
           __builtin_amdgcn_sched_barrier(0);  // behind the products above
           uint32_t kn[NKA];
@@ -1117,8 +1147,10 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
       return score_step((uint32_t)ring * G::STAGE, cc);  // large body: a single copy keeps the kernel in the instruction cache
     }
   };
-  auto run_score_step_pre = [&](int ring, bool more) __attribute__((always_inline)) -> bool {
-    return score_step((uint32_t)ring * G::STAGE, cc, more ? (uint32_t)((ring + 1) & (NS - 1)) * G::STAGE : 0xffffffffu);
+  auto run_score_step_pre = [&](int ring, bool more) __attribute__((always_inline)) -> bool {  // more: the step has another tile
+    // (one copy of the body with a run-time slot offset, also for one row block: with the operands carried across four
+    // copies the compiler spills)
+    return score_step((uint32_t)ring * G::STAGE, cc, (uint32_t)((ring + 1) & (NS - 1)) * G::STAGE, more);
   };
   int u = 0, ring = 0, seg_count = 0;
   // two waves per SIMD: the accumulators are ordinary vector registers, the rescale can sit in the loop
@@ -1160,7 +1192,7 @@ __global__ __launch_bounds__(NW * 64, (SHW > 1 && (D <= 128 || SHW == 8)) ? 2 : 
 #pragma nounroll
         for (int sub = 0; sub < step; ++sub) {  // (a loop, not two copies: the body is large)
           bool moved_;
-          if constexpr (KPRE) moved_ = run_score_step_pre(ring, sub + 1 < step);
+          if constexpr (KPRE || KPRE2) moved_ = run_score_step_pre(ring, sub + 1 < step);
           else moved_ = run_score_step(ring);
           if (__builtin_expect(moved_, 0)) rescale();
           value_step((uint32_t)ring * G::STAGE);
